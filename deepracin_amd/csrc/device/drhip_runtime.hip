@@ -1,0 +1,119 @@
+// Device bring-up, streams, events and memory of the HIP device layer (see include/dr_hip.h).
+#include "drhip_common.hpp"
+
+#include <cstring>
+
+namespace drhip {
+
+char* error_slot() {
+    static thread_local char msg[512] = "no error";
+    return msg;
+}
+
+static int g_num_cu = 256;
+int num_cu() { return g_num_cu; }
+
+__global__ void fill_f32_kernel(float* __restrict__ dst, float value, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = value;
+}
+
+}  // namespace drhip
+
+using namespace drhip;
+
+extern "C" {
+
+const char* drhip_last_error(void) { return error_slot(); }
+
+int drhip_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; }
+    return n;
+}
+
+int drhip_init(int device, drhip_device_info* info) {
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return fail(DRHIP_ENODEVICE, "no HIP device available (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+    }
+    DRHIP_REQUIRE(device >= 0 && device < n, "device ordinal %d out of range [0,%d)", device, n);
+    if (int rc = check(hipSetDevice(device), "hipSetDevice")) return rc;
+    hipDeviceProp_t p;
+    if (int rc = check(hipGetDeviceProperties(&p, device), "hipGetDeviceProperties")) return rc;
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
+        return fail(DRHIP_ENODEVICE, "device %d is %s; this library carries gfx950 code only", device, p.gcnArchName);
+    g_num_cu = p.multiProcessorCount;
+    if (info) {
+        memset(info, 0, sizeof(*info));
+        strncpy(info->name, p.name, sizeof(info->name) - 1);
+        strncpy(info->arch, p.gcnArchName, sizeof(info->arch) - 1);
+        info->device = device;
+        info->num_cu = p.multiProcessorCount;
+        info->wavefront = p.warpSize;
+        info->lds_bytes = (int)p.sharedMemPerBlock;
+        info->clock_khz = p.clockRate;
+        info->hbm_bytes = p.totalGlobalMem;
+        info->l2_bytes = p.l2CacheSize;
+    }
+    return DRHIP_OK;
+}
+
+int drhip_stream_create(void** stream) {
+    DRHIP_REQUIRE(stream, "stream out-pointer is NULL");
+    hipStream_t s;
+    if (int rc = check(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreate")) return rc;
+    *stream = (void*)s;
+    return DRHIP_OK;
+}
+int drhip_stream_destroy(void* stream) { return stream ? check(hipStreamDestroy(as_stream(stream)), "hipStreamDestroy") : DRHIP_OK; }
+int drhip_stream_sync(void* stream) { return check(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize"); }
+
+int drhip_event_create(void** ev) {
+    DRHIP_REQUIRE(ev, "event out-pointer is NULL");
+    hipEvent_t e;
+    if (int rc = check(hipEventCreate(&e), "hipEventCreate")) return rc;
+    *ev = (void*)e;
+    return DRHIP_OK;
+}
+int drhip_event_destroy(void* ev) { return ev ? check(hipEventDestroy((hipEvent_t)ev), "hipEventDestroy") : DRHIP_OK; }
+int drhip_event_record(void* ev, void* stream) { return check(hipEventRecord((hipEvent_t)ev, as_stream(stream)), "hipEventRecord"); }
+int drhip_event_elapsed_ms(void* a, void* b, float* ms) {
+    DRHIP_REQUIRE(a && b && ms, "NULL event or result pointer");
+    if (int rc = check(hipEventSynchronize((hipEvent_t)b), "hipEventSynchronize")) return rc;
+    return check(hipEventElapsedTime(ms, (hipEvent_t)a, (hipEvent_t)b), "hipEventElapsedTime");
+}
+
+int drhip_malloc(void** dptr, size_t bytes) {
+    DRHIP_REQUIRE(dptr && bytes > 0, "drhip_malloc: NULL out-pointer or zero size");
+    return check(hipMalloc(dptr, bytes), "hipMalloc");
+}
+int drhip_free(void* dptr) { return dptr ? check(hipFree(dptr), "hipFree") : DRHIP_OK; }
+
+int drhip_upload(void* dst, size_t off, const void* src, size_t bytes, void* stream) {
+    DRHIP_REQUIRE(dst && src, "drhip_upload: NULL pointer");
+    if (bytes == 0) return DRHIP_OK;
+    if (int rc = check(hipMemcpyAsync((char*)dst + off, src, bytes, hipMemcpyHostToDevice, as_stream(stream)), "hipMemcpyAsync(H2D)")) return rc;
+    return check(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize(H2D)");
+}
+int drhip_download(void* dst, const void* src, size_t off, size_t bytes, void* stream) {
+    DRHIP_REQUIRE(dst && src, "drhip_download: NULL pointer");
+    if (bytes == 0) return DRHIP_OK;
+    if (int rc = check(hipMemcpyAsync(dst, (const char*)src + off, bytes, hipMemcpyDeviceToHost, as_stream(stream)), "hipMemcpyAsync(D2H)")) return rc;
+    return check(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize(D2H)");
+}
+
+int drhip_fill_f32(float* dst, float value, size_t n, void* stream) {
+    DRHIP_REQUIRE(dst, "drhip_fill_f32: NULL pointer");
+    if (n == 0) return DRHIP_OK;
+    const int block = 256;
+    size_t blocks = (n + block - 1) / block;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)blocks), dim3(block), 0, as_stream(stream), dst, value, n);
+    return launched("fill_f32_kernel");
+}
+
+}  // extern "C"

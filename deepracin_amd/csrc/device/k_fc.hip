@@ -1,0 +1,184 @@
+// Fully connected layer at batch 1 = GEMV y[n] = act(b[n] + sum_k x[k] * Wt[k][n]); HBM-bound:
+// algorithmic bytes = 4*(K*N + K + 2N), every weight is read exactly once.
+//
+// Mapping for gfx950
+//   - Wt is [K][N], n fastest, so one row segment is contiguous: a wavefront reads 64 x float4 =
+//     1 KiB of one row per load instruction (fully coalesced, nontemporal: the matrix is streamed
+//     once and must not evict activations from L2 / Infinity Cache);
+//   - a workgroup (4 waves) owns a panel of CBW = 64*VEC columns and a slice of rows; its waves take
+//     64-row chunks round-robin and keep 8 row loads in flight per lane;
+//   - x for a 64-row chunk is loaded once, one element per lane, and broadcast with v_readlane;
+//   - split-K: the grid is (column panels) x (row slices), sized to a few workgroups per CU; each
+//     workgroup writes one partial row, the LAST workgroup of a panel to arrive (device-scope
+//     counter) sums the partials in slice order, adds the bias, applies ReLU and resets the
+//     counter.  Summation order is fixed, so results are reproducible run to run.
+//
+// Reference semantics: Kernels/dR_fcl.cl:59-120 (two kernels: partial sums over partitions of K,
+// then a sequential sum of the partials + bias + clamp).  The partition size there depends on the
+// OpenCL device; any partitioning gives the same sum up to fp32 rounding.
+#include "drhip_common.hpp"
+
+namespace drhip {
+
+constexpr int kFcThreads = 256;
+constexpr int kFcWaves = kFcThreads / kWave;
+constexpr int kFcUnroll = 8;
+
+template <int VEC> struct VecT;
+template <> struct VecT<4> { typedef float __attribute__((ext_vector_type(4))) type; };
+template <> struct VecT<2> { typedef float __attribute__((ext_vector_type(2))) type; };
+template <> struct VecT<1> { typedef float type; };
+
+template <int VEC>
+__device__ inline void fma_row(float (&acc)[VEC], const typename VecT<VEC>::type& w, float xv) {
+    if constexpr (VEC == 1) acc[0] = fmaf(w, xv, acc[0]);
+    else {
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) acc[v] = fmaf(w[v], xv, acc[v]);
+    }
+}
+
+struct FcPlan { int vec, cbw, panels, slices, rowsPerSlice; };
+
+// Split of the [K][N] matrix into column panels and row slices.
+static FcPlan fc_plan(int K, int N) {
+    FcPlan p;
+    p.vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+    p.cbw = kWave * p.vec;
+    p.panels = ceil_div(N, p.cbw);
+    const int target = 4 * num_cu();                 // workgroups wanted in flight
+    int slices = ceil_div(target, p.panels);
+    const int maxSlices = ceil_div(K, 2 * kWave);    // at least two 64-row chunks per workgroup
+    if (slices > maxSlices) slices = maxSlices;
+    if (slices < 1) slices = 1;
+    p.rowsPerSlice = ceil_div(ceil_div(K, slices), kWave) * kWave;   // whole chunks
+    p.slices = ceil_div(K, p.rowsPerSlice);
+    return p;
+}
+
+template <int VEC>
+__global__ void __launch_bounds__(kFcThreads)
+fc_gemv_kernel(const float* __restrict__ x, const float* __restrict__ Wt, const float* __restrict__ bias,
+               float* __restrict__ y, float* __restrict__ partials, int* __restrict__ counters,
+               int K, int N, int rowsPerSlice, int relu) {
+    typedef typename VecT<VEC>::type vec_t;
+    constexpr int CBW = kWave * VEC;
+    __shared__ float red[kFcWaves][CBW];
+    __shared__ int amLast;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int panel = blockIdx.x, slice = blockIdx.y, slices = gridDim.y;
+    const int col = panel * CBW + lane * VEC;
+    const bool colOk = col < N;                      // N % VEC == 0, so a vector is all-in or all-out
+    const int rowBegin = slice * rowsPerSlice;
+    const int rowEnd = min(K, rowBegin + rowsPerSlice);
+
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
+
+    for (int r0 = rowBegin + wave * kWave; r0 < rowEnd; r0 += kFcWaves * kWave) {
+        const int rows = min(kWave, rowEnd - r0);
+        const float xl = (lane < rows) ? x[r0 + lane] : 0.0f;
+        const float* wp = Wt + (size_t)r0 * N + col;
+        if (rows == kWave) {
+#pragma unroll
+            for (int j0 = 0; j0 < kWave; j0 += kFcUnroll) {
+                vec_t w[kFcUnroll];
+#pragma unroll
+                for (int u = 0; u < kFcUnroll; ++u)
+                    if (colOk) w[u] = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)(j0 + u) * N));
+#pragma unroll
+                for (int u = 0; u < kFcUnroll; ++u)
+                    if (colOk) fma_row<VEC>(acc, w[u], __builtin_amdgcn_readlane(xl, j0 + u));
+            }
+        } else {
+            for (int j = 0; j < rows; ++j) {
+                const float xv = __shfl(xl, j, 64);
+                if (colOk) {
+                    vec_t w = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)j * N));
+                    fma_row<VEC>(acc, w, xv);
+                }
+            }
+        }
+    }
+
+    // combine the four waves of the workgroup
+#pragma unroll
+    for (int v = 0; v < VEC; ++v) red[wave][lane * VEC + v] = acc[v];
+    __syncthreads();
+    const int ncols = min(CBW, N - panel * CBW);
+    for (int c = tid; c < ncols; c += kFcThreads) {
+        float s = red[0][c];
+#pragma unroll
+        for (int w = 1; w < kFcWaves; ++w) s += red[w][c];
+        partials[(size_t)slice * N + panel * CBW + c] = s;
+    }
+
+    // last workgroup of this panel finishes the sum
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) amLast = (atomicAdd(&counters[panel], 1) == slices - 1);
+    __syncthreads();
+    if (!amLast) return;
+    __threadfence();
+    for (int c = tid; c < ncols; c += kFcThreads) {
+        const int n = panel * CBW + c;
+        float s = 0.0f;
+        for (int sl = 0; sl < slices; ++sl) s += __builtin_nontemporal_load(&partials[(size_t)sl * N + n]);
+        if (bias) s += bias[n];
+        if (relu) s = fmaxf(s, 0.0f);
+        y[n] = s;
+    }
+    if (tid == 0) counters[panel] = 0;
+}
+
+__global__ void __launch_bounds__(256)
+fc_permute_rows_kernel(const float* __restrict__ src, float* __restrict__ dst, int W, int H, int C, int N) {
+    // one workgroup per destination row k_chw = (z*H + y)*W + x  <-  source row k_hwc = (y*W + x)*C + z
+    const int k = blockIdx.x;
+    const int x = k % W, y = (k / W) % H, z = k / (W * H);
+    const size_t srow = ((size_t)(y * W + x) * C + z) * N, drow = (size_t)k * N;
+    for (int n = threadIdx.x; n < N; n += blockDim.x) dst[drow + n] = src[srow + n];
+}
+
+}  // namespace drhip
+
+using namespace drhip;
+
+extern "C" size_t drhip_fc_scratch_floats(int K, int N) {
+    if (K <= 0 || N <= 0) return 0;
+    FcPlan p = fc_plan(K, N);
+    return (size_t)p.slices * (size_t)N;
+}
+
+extern "C" size_t drhip_fc_scratch_counters(int K, int N) {
+    if (K <= 0 || N <= 0) return 0;
+    return (size_t)fc_plan(K, N).panels;
+}
+
+extern "C" int drhip_fc_f32(const float* x, const float* Wt, const float* bias, float* y,
+                            float* partials, int* counters, int K, int N, int relu, void* stream) {
+    DRHIP_REQUIRE(x && Wt && y && partials && counters, "drhip_fc_f32: NULL pointer");
+    DRHIP_REQUIRE(K > 0 && N > 0, "drhip_fc_f32: bad shape K=%d N=%d", K, N);
+    FcPlan p = fc_plan(K, N);
+    DRHIP_REQUIRE(((size_t)Wt % (4 * p.vec)) == 0, "drhip_fc_f32: weight matrix not aligned for %d-wide loads", p.vec);
+    DRHIP_REQUIRE(p.slices <= 65535, "drhip_fc_f32: too many row slices");
+    dim3 grid(p.panels, p.slices), block(kFcThreads);
+    hipStream_t s = as_stream(stream);
+    if (p.vec == 4)
+        hipLaunchKernelGGL((fc_gemv_kernel<4>), grid, block, 0, s, x, Wt, bias, y, partials, counters, K, N, p.rowsPerSlice, relu);
+    else if (p.vec == 2)
+        hipLaunchKernelGGL((fc_gemv_kernel<2>), grid, block, 0, s, x, Wt, bias, y, partials, counters, K, N, p.rowsPerSlice, relu);
+    else
+        hipLaunchKernelGGL((fc_gemv_kernel<1>), grid, block, 0, s, x, Wt, bias, y, partials, counters, K, N, p.rowsPerSlice, relu);
+    return launched("fc_gemv_kernel");
+}
+
+extern "C" int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, int H, int C, int N, void* stream) {
+    DRHIP_REQUIRE(src && dst && src != dst, "drhip_fc_permute_rows_f32: NULL or aliased matrices");
+    DRHIP_REQUIRE(W > 0 && H > 0 && C > 0 && N > 0, "drhip_fc_permute_rows_f32: bad shape");
+    DRHIP_REQUIRE((long long)W * H * C < (1ll << 31), "drhip_fc_permute_rows_f32: K too large");
+    hipLaunchKernelGGL(fc_permute_rows_kernel, dim3(W * H * C), dim3(256), 0, as_stream(stream), src, dst, W, H, C, N);
+    return launched("fc_permute_rows_kernel");
+}

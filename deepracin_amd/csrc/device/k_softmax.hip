@@ -1,0 +1,70 @@
+// Softmax over a flat fp32 vector in ONE workgroup: wavefront-level butterfly reductions
+// (ds_bpermute via __shfl_xor) for max and sum, one small LDS exchange between the waves.
+//
+// The reference computes exp(x) on the device, downloads the vector, sums it sequentially on the
+// host and launches a scale kernel (src/dR_nodes_math.c:620-678).  Mathematically this kernel is
+// the same function, exp(x_i)/sum_j exp(x_j); it subtracts max(x) first so that large logits do
+// not overflow, and the whole node stays on the device and asynchronous.
+#include "drhip_common.hpp"
+
+#include <cfloat>
+
+namespace drhip {
+
+constexpr int kSoftmaxThreads = 1024;
+
+__device__ inline float wave_max(float v) {
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ inline float wave_sum(float v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__global__ void __launch_bounds__(kSoftmaxThreads)
+softmax_kernel(const float* __restrict__ x, float* __restrict__ y, int n) {
+    __shared__ float red[kSoftmaxThreads / kWave];
+    __shared__ float bcast;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int nwaves = kSoftmaxThreads / kWave;
+
+    float m = -FLT_MAX;
+    for (int i = tid; i < n; i += kSoftmaxThreads) m = fmaxf(m, x[i]);
+    m = wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    if (wave == 0) {
+        float v = lane < nwaves ? red[lane] : -FLT_MAX;
+        v = wave_max(v);
+        if (lane == 0) bcast = v;
+    }
+    __syncthreads();
+    m = bcast;
+
+    float s = 0.0f;
+    for (int i = tid; i < n; i += kSoftmaxThreads) s += expf(x[i] - m);
+    s = wave_sum(s);
+    __syncthreads();            // everyone has read bcast / red from the first round
+    if (lane == 0) red[wave] = s;
+    __syncthreads();
+    if (wave == 0) {
+        float v = lane < nwaves ? red[lane] : 0.0f;
+        v = wave_sum(v);
+        if (lane == 0) bcast = 1.0f / v;
+    }
+    __syncthreads();
+    const float inv = bcast;
+    for (int i = tid; i < n; i += kSoftmaxThreads) y[i] = expf(x[i] - m) * inv;
+}
+
+}  // namespace drhip
+
+using namespace drhip;
+
+extern "C" int drhip_softmax_f32(const float* x, float* y, int n, void* stream) {
+    DRHIP_REQUIRE(x && y, "drhip_softmax_f32: NULL tensor");
+    DRHIP_REQUIRE(n > 0, "drhip_softmax_f32: n = %d", n);
+    hipLaunchKernelGGL(softmax_kernel, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, y, n);
+    return launched("softmax_kernel");
+}

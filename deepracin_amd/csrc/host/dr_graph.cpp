@@ -1,0 +1,310 @@
+// Graph life cycle of the deepRacin C API on top of the HIP device layer:
+// dR_NewGraph / dR_config / dR_initCL / dR_prepare / dR_apply / dR_feedData / dR_getOutputBuffers /
+// dR_downloadArray / dR_cleanup.  Same call contract as the reference's src/deepRACIN.c and the
+// buffer helpers of src/dR_clwrap.c; everything underneath is HIP.
+#include "dr_internal.hpp"
+
+#include <chrono>
+
+using namespace dr;
+
+extern "C" {
+
+// Defaults as in the reference (src/deepRACIN.c:6-47): silent, no profiling, first GPU.
+dR_Graph* dR_NewGraph(void) {
+    dR_Graph* g = zalloc<dR_Graph>();
+    g->clConfig = zalloc<dR_ClConfig>();
+    g->config = zalloc<dR_Config>();
+
+    dR_ClConfig* cc = g->clConfig;
+    cc->clEvent = &cc->clEventObject;
+    cc->clDeviceType = CL_DEVICE_TYPE_GPU;
+    cc->clDeviceNumber = 0;
+    cc->clInfo = TRUE;
+    cc->clKernelPath = (gchar*)"";
+    cc->clPlatformName = (gchar*)" ";
+    cc->fastRelaxedMath = TRUE;
+    cc->forceRecompile = TRUE;
+
+    g->config->silent = TRUE;
+
+    g->feed_layers = dR_list_createEmptyList();
+    g->output_layers = dR_list_createEmptyList();
+    g->allNodes = dR_list_createEmptyList();
+    g->drViewHandlers = dR_list_createEmptyList();
+    g->debugLayer = -1;     // the reference leaves this uninitialised; -1 = no debug download
+    return g;
+}
+
+void dR_config(dR_Graph* net, gchar* platformname, gboolean silent, gboolean debuginfo,
+               gboolean profileGPU, gboolean profileCPU, gchar* temppath) {
+    net->clConfig->clPlatformName = platformname ? strdup(platformname) : NULL;
+    net->config->silent = silent;
+    net->config->debugInfo = debuginfo;
+    net->config->profilingCPU = profileCPU;
+    net->config->profilingGPU = profileGPU;
+    net->config->modelPath = temppath;
+}
+
+// Bring up the HIP device and the graph's stream.  Idempotent.
+static gboolean ensure_device(dR_Graph* net) {
+    dR_ClConfig* cc = net->clConfig;
+    if (cc->clContext) return TRUE;
+    drhip_device_info info;
+    if (device_failed(net, drhip_init((int)cc->clDeviceNumber, &info), "dR_initCL")) return FALSE;
+    if (!cc->hipStream) {
+        if (device_failed(net, drhip_stream_create(&cc->hipStream), "dR_initCL(stream)")) return FALSE;
+        cc->hipOwnsStream = TRUE;
+    }
+    cc->clCommandQueue = (cl_command_queue)cc->hipStream;
+    cc->clDeviceName = fmt_dup("%s (%s)", info.name, info.arch);
+    cc->hipNumCU = info.num_cu;
+    cc->hipLdsBytes = info.lds_bytes;
+    cc->clNumDevices = 1;
+    cc->clContext = (cl_context)cc;     // tag: device is up
+    if (verbose(net))
+        say("deepRACIN HIP device %d: %s, %d CUs, %d KiB LDS/workgroup, %.1f GiB HBM\n", info.device,
+            cc->clDeviceName, info.num_cu, info.lds_bytes / 1024, (double)info.hbm_bytes / (1 << 30));
+    return TRUE;
+}
+
+void dR_initCL(dR_Graph* net) { ensure_device(net); }
+
+void dR_setClEnvironment(dR_Graph* net, cl_context, cl_platform_id, cl_command_queue clcommandqueue,
+                         cl_device_id) {
+    // The only thing a HIP caller can share is its stream.
+    net->clConfig->hipStream = (void*)clcommandqueue;
+    net->clConfig->hipOwnsStream = FALSE;
+}
+
+void dR_getClEnvironmentFrom(dR_Graph* net, dR_Graph* from) {
+    if (!from || !from->clConfig->clContext) return;
+    net->clConfig->hipStream = from->clConfig->hipStream;
+    net->clConfig->hipOwnsStream = FALSE;
+    net->clConfig->clDeviceNumber = from->clConfig->clDeviceNumber;
+}
+
+gboolean dR_setAsOutput(dR_Graph* net, dR_Node* node) {
+    if (!node->output) {
+        node->output = TRUE;
+        dR_list_append(net->output_layers, node);
+    }
+    return TRUE;
+}
+
+gboolean dR_prepare(dR_Graph* net) {
+    const bool talk = verbose(net);
+    if (!ensure_device(net)) { say("dR_initCL Failed \n"); return FALSE; }
+
+    if (talk) say("Propagate shapes and schedule...\n");
+    if (!dR_propagateShapesAndSchedule(net)) { say("dR_propagateShapesAndSchedule Failed \n"); return FALSE; }
+    if (talk) say("Done.\n");
+
+    if (talk) say("Select kernels...\n");
+    if (!dR_generateAndCompileKernels(net)) { say("\ndR_generateAndCompileKernels Failed \n"); return FALSE; }
+    if (talk) say("Done.\n");
+
+    if (talk) say("Estimate and allocate buffers...\n");
+    if (!dR_estimateAndAllocateBuffers(net)) { say("dR_estimateAndAllocateBuffers Failed \n"); return FALSE; }
+    if (talk) say("Done. \n");
+
+    if (talk) say("Fill buffers...\n");
+    if (!dR_fillBuffers(net)) { say("dR_fillBuffers Failed \n"); return FALSE; }
+    if (device_failed(net, drhip_stream_sync(stream_of(net)), "dR_prepare(sync)")) return FALSE;
+    if (talk) say("Done.\n\n");
+
+    net->prepared = TRUE;
+    if (net->config->profilingGPU) {
+        say("\nGPU Profiling: Whole graph GPU memory consumption: %4.6f MB \n\n",
+            (double)net->clConfig->memConsumptionGPU / 1048576.0);
+        net->clConfig->totalKernelGPUTime = 0;
+    }
+    return TRUE;
+}
+
+gint dR_getOutputBuffers(dR_Graph* net, cl_mem** outptr) {
+    if (!net->prepared) {
+        say("dR_Graph must be prepared before having output buffers. Call dR_prepare first! \n");
+        return 0;
+    }
+    int n = 0;
+    for (dR_ListElement* e = net->output_layers->first; e && n < 10; e = e->next)
+        outptr[n++] = ((dR_Node*)e->element)->outputBuf->bufptr;
+    return n;
+}
+
+void dR_feedData(dR_Graph* net, dR_Node* feednode, gfloat* data, gint offset, gint numfloats) {
+    dR_uploadArray(net, (gchar*)"", data, (size_t)offset * sizeof(float), (size_t)numfloats * sizeof(float),
+                   feednode->outputBuf->buf);
+}
+
+// One forward pass: walks the schedule and lets every node enqueue its kernels.  Asynchronous
+// unless profiling is enabled (reference src/deepRACIN.c:204-270: clFlush only).
+//
+// profilingGPU: the reference waits for every kernel and reads its cl_event (src/dR_clwrap.c:970-1049).
+// Here one hipEvent is recorded between consecutive nodes while the whole pass is enqueued without
+// waiting; after the last node the pass is awaited once and the differences of neighbouring events
+// give each node's device time (node->drLastKernelMs) and their sum (clConfig->totalKernelGPUTime,
+// printed like the reference does).  The stream therefore runs at its natural pace and the times
+// are not inflated by host launch latency.
+gboolean dR_apply(dR_Graph* net) {
+    if (!net->prepared) { say("dR_apply: graph is not prepared. Call dR_prepare first! \n"); return FALSE; }
+    dR_ClConfig* cc = net->clConfig;
+    const bool profGPU = net->config->profilingGPU, profCPU = net->config->profilingCPU;
+    if (net->config->debugInfo) say("Applying graph...\n");
+
+    std::chrono::steady_clock::time_point t0;
+    if (profCPU) { t0 = std::chrono::steady_clock::now(); net->config->totalNodeCPUTime = 0.0; }
+
+    const int nNodes = net->scheduledLayers->length;
+    if (profGPU && cc->hipNumEvents < nNodes + 1) {
+        void** ev = (void**)realloc(cc->hipEvents, sizeof(void*) * (size_t)(nNodes + 1));
+        if (!ev) return FALSE;
+        cc->hipEvents = ev;
+        for (; cc->hipNumEvents < nNodes + 1; cc->hipNumEvents++)
+            if (device_failed(net, drhip_event_create(&cc->hipEvents[cc->hipNumEvents]), "dR_apply(profile)")) return FALSE;
+    }
+    if (profGPU) drhip_event_record(cc->hipEvents[0], cc->hipStream);
+
+    int pos = 0;
+    for (dR_ListElement* e = net->scheduledLayers->first; e; e = e->next, ++pos) {
+        dR_Node* node = (dR_Node*)e->element;
+        if (!node->compute(net, node)) {
+            say("Execution of layer %d failed \n", node->layerID);
+            return FALSE;
+        }
+        if (profGPU) drhip_event_record(cc->hipEvents[pos + 1], cc->hipStream);
+        if (node->layerID == net->debugLayer && net->hostDebugBuffer)
+            dR_downloadArray(net, (gchar*)"", node->outputBuf->bufptr, 0,
+                             (size_t)node->oshape.s0 * node->oshape.s1 * sizeof(float), net->hostDebugBuffer);
+    }
+    if (profGPU) {
+        pos = 0;
+        cc->totalKernelGPUTime = 0;
+        for (dR_ListElement* e = net->scheduledLayers->first; e; e = e->next, ++pos) {
+            float ms = 0.f;
+            if (device_failed(net, drhip_event_elapsed_ms(cc->hipEvents[pos], cc->hipEvents[pos + 1], &ms), "dR_apply(profile)"))
+                return FALSE;
+            ((dR_Node*)e->element)->drLastKernelMs = ms;
+            cc->totalKernelGPUTime += ms;
+        }
+        say("GPU Profiling: Sum of all kernel run times: %2.3fms \n", cc->totalKernelGPUTime);   // unconditional, like the reference
+        cc->sumTotalKernelGPUTime += cc->totalKernelGPUTime;
+        if (cc->totalKernelGPUTime > cc->maxTotalKernelGPUTime) cc->maxTotalKernelGPUTime = cc->totalKernelGPUTime;
+        cc->queueKernelGPUTime = cc->totalKernelGPUTime;   // last pass, kept after the running sum is reset
+        cc->totalKernelGPUTime = 0;
+    }
+    if (profCPU) {
+        if (device_failed(net, drhip_stream_sync(cc->hipStream), "dR_apply(sync)")) return FALSE;
+        double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        net->drLastApplyMs = ms;
+        say("CPU Profiling: Whole graph took: %2.3fms, Sum of all nodes: %2.3fms \n", ms, net->config->totalNodeCPUTime);
+    }
+    if (net->config->debugInfo) say("Done.\n\n");
+    return TRUE;
+}
+
+void dR_cleanup(dR_Graph* net, gboolean cleanupcl) {
+    const bool talk = verbose(net);
+    if (talk) say("Cleaning up deepRACIN...\n");
+    if (net->clConfig->clContext) drhip_stream_sync(net->clConfig->hipStream);
+    if (net->prepared) dR_cleanupBuffers(net);
+    if (cleanupcl) dR_cleanupCL(net);
+    dR_cleanupNet(net);
+    if (talk) say("Done.\n");
+}
+
+gboolean dR_cleanupCL(dR_Graph* net) {
+    dR_ClConfig* cc = net->clConfig;
+    if (!cc->clContext || cc->cleanupDone) return TRUE;
+    for (int i = 0; i < cc->hipNumEvents; ++i) drhip_event_destroy(cc->hipEvents[i]);
+    free(cc->hipEvents);
+    cc->hipEvents = NULL;
+    cc->hipNumEvents = 0;
+    if (cc->hipOwnsStream && cc->hipStream) drhip_stream_destroy(cc->hipStream);
+    cc->hipStream = NULL;
+    free(cc->clDeviceName);
+    cc->clDeviceName = NULL;
+    cc->clContext = NULL;
+    cc->cleanupDone = TRUE;
+    return TRUE;
+}
+
+gboolean dR_saveGraph(dR_Graph* net, gchar* path) { return dR_serializeGraph(net, path); }
+
+dR_Node* dR_loadGraph(dR_Graph* net, gchar* path, dR_Node*** nodelist, gint* numnodes,
+                      dR_Node*** feednodes, gint* numfeednodes) {
+    return dR_parseGraph(net, path, nodelist, numnodes, feednodes, numfeednodes);
+}
+
+void dR_printNetObject(dR_Graph* net, char* path) { dR_printNet(net, path); }
+
+dR_Shape3* dR_getOutputShape(dR_Node* node) { return &node->oshape; }
+
+dR_Shape3* dR_getFeedNodeInputShape(dR_Node* node) {
+    if (node->type != tDataFeedNode) {
+        say("Error: dR_getFeedNodeInputShape only works on feed nodes!\n");
+        return NULL;
+    }
+    return &((dR_DataFeedNode_Data*)node->layer)->shape;
+}
+
+// ---- caller-supplied buffers -------------------------------------------------------------------
+
+gboolean dR_setDataFeedNodeBuffer(dR_Graph* net, dR_Node* node, cl_mem* buf) {
+    if (node->type != tDataFeedNode) {
+        if (verbose(net)) say("dR_setDataFeedNodeBuffer Error: Data Feed Buffer can only be set to a DataFeedNode!\n");
+        return FALSE;
+    }
+    dR_DataFeedNode_Data* feed = (dR_DataFeedNode_Data*)node->layer;
+    node->outputBuf = dR_newMemoryHandler(TRUE);
+    node->outputBuf->bufptr = buf;
+    node->outputBuf->buf = *buf;
+    node->outputBuf->size = feed->shape.s0 * feed->shape.s1 * feed->shape.s2;
+    dR_list_append(node->outputBuf->outputFor, node);
+    return TRUE;
+}
+
+gboolean dR_setPreexistingOutputBuffer(dR_Graph* net, dR_Node* node, cl_mem* buf) {
+    node->outputBuf = dR_newMemoryHandler(TRUE);
+    node->outputBuf->bufptr = buf;
+    node->outputBuf->buf = *buf;
+    if (!node->output) dR_setAsOutput(net, node);
+    return TRUE;
+}
+
+// Region-of-interest plumbing belongs to the image-processing nodes, which this build does not carry.
+gboolean dR_setNodeRoI(dR_Node*, dR_Shape3) { return FALSE; }
+gboolean dR_setNodeRoIBufferAndIndex(dR_Node*, cl_mem*, gint) { return FALSE; }
+
+// ---- device memory helpers (names of the reference's OpenCL wrapper) ------------------------------
+
+gboolean dR_createFloatBuffer(dR_Graph* net, cl_mem* mem, gint size, int /*buffertype*/) {
+    if (size <= 0) { say("dR_createFloatBuffer: refusing to allocate %d floats\n", size); return FALSE; }
+    void* p = NULL;
+    if (device_failed(net, drhip_malloc(&p, (size_t)size * sizeof(float)), "dR_createFloatBuffer")) return FALSE;
+    *mem = (cl_mem)p;
+    net->clConfig->memConsumptionGPU += (glong)size * (glong)sizeof(float);
+    return TRUE;
+}
+
+gboolean dR_clMemoryBufferCleanup(dR_Graph* net, cl_mem mem) {
+    if (!mem) return TRUE;
+    return !device_failed(net, drhip_free((void*)mem), "dR_clMemoryBufferCleanup");
+}
+
+gboolean dR_uploadArray(dR_Graph* net, gchar*, void* srcHostMem, size_t offset, size_t numBytes,
+                        cl_mem destDeviceMem) {
+    if (!destDeviceMem || !srcHostMem) { say("dR_uploadArray: NULL buffer\n"); return FALSE; }
+    return !device_failed(net, drhip_upload((void*)destDeviceMem, offset, srcHostMem, numBytes, stream_of(net)),
+                          "dR_uploadArray");
+}
+
+void dR_downloadArray(dR_Graph* net, gchar*, cl_mem* srcDeviceMem, size_t byteOffset, size_t numBytes,
+                      void* destHostMem) {
+    if (!srcDeviceMem || !*srcDeviceMem || !destHostMem) { say("dR_downloadArray: NULL buffer\n"); return; }
+    device_failed(net, drhip_download(destHostMem, (const void*)*srcDeviceMem, byteOffset, numBytes, stream_of(net)),
+                  "dR_downloadArray");
+}
+
+}  // extern "C"

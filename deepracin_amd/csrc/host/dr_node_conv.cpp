@@ -1,0 +1,236 @@
+// Conv2d node: constructor, graph.dr (de)serialisation, and the three gfx950 execution paths.
+//
+// Node contract = reference src/dR_nodes_conv2d.c:12-256 (constructor, shape rule out = in/stride,
+// 10 parameters + 1..2 variables in graph.dr, deep copy in setVariables).  What differs is below the
+// vtable: schedule() assigns a HIP kernel variant instead of OpenCL work sizes, fillBuffers() uploads
+// weights in the layout that kernel streams best, compute() enqueues through drhip_*.
+#include "dr_internal.hpp"
+
+using namespace dr;
+
+namespace {
+
+inline dR_Conv2d_Data* conv_of(dR_Node* n) { return (dR_Conv2d_Data*)n->layer; }
+inline int weight_count(const dR_Conv2d_Data* c) { return c->shape.s0 * c->shape.s1 * c->shape.s2 * c->shape.s3; }
+
+gboolean conv_propagate(dR_Graph* net, dR_Node* node) {
+    dR_Conv2d_Data* c = conv_of(node);
+    if (node->previous_layers->length != 1 && verbose(net))
+        say("Conv2d Layer with id %d has %d inputs but needs 1!\n", node->layerID, node->previous_layers->length);
+    dR_Node* in = first_input(node);
+    if (!in) return FALSE;
+    c->ishape = in->oshape;
+    if (c->stride.s1 <= 0 || c->stride.s2 <= 0) { say("Conv2d stride must be positive! \n"); return FALSE; }
+    node->oshape.s0 = c->ishape.s0 / c->stride.s1;
+    node->oshape.s1 = c->ishape.s1 / c->stride.s2;
+    node->oshape.s2 = c->shape.s3;
+    if (node->oshape.s0 <= 0 || node->oshape.s1 <= 0 || node->oshape.s2 <= 0) {
+        say("Conv2d shape propagates to Zero. False shape parameters! \n");
+        return FALSE;
+    }
+    if (c->ishape.s2 != c->shape.s2) {
+        say("Conv2d Layer %d expects %d input channels but its input has %d! \n", node->layerID, c->shape.s2, c->ishape.s2);
+        return FALSE;
+    }
+    return TRUE;
+}
+
+gint32 conv_out_size(dR_Node* node) { return node->oshape.s0 * node->oshape.s1 * node->oshape.s2; }
+
+gchar* conv_serialize(dR_Node* node, gchar* params[], gint* numParams, gfloat* variables[], gint variableSizes[],
+                      gint* numVariables) {
+    dR_Conv2d_Data* c = conv_of(node);
+    const int needVars = c->useBias ? 2 : 1;
+    if (*numParams < 10 || *numVariables < needVars) {
+        say("SerializeNode needs space for %d parameters and %d variables!\n", 10, needVars);
+        return NULL;
+    }
+    const int vals[10] = { (int)c->activation, c->useBias ? 1 : 0, c->shape.s0, c->shape.s1, c->shape.s2, c->shape.s3,
+                           c->stride.s0, c->stride.s1, c->stride.s2, c->stride.s3 };
+    for (int i = 0; i < 10; ++i) params[i] = fmt_dup("%d", vals[i]);
+    *numParams = 10;
+    *numVariables = needVars;
+    variableSizes[0] = weight_count(c);
+    variables[0] = c->weights;
+    if (c->useBias) { variableSizes[1] = c->shape.s3; variables[1] = c->biases; }
+    return (gchar*)"Conv2D";
+}
+
+gchar* conv_print(dR_Node* node) {
+    dR_Conv2d_Data* c = conv_of(node);
+    static const char* acts[] = { "Linear", "ReLU", "Sigmoid", "Tan" };
+    static const char* algos[] = { "direct", "Winograd F(2x2,3x3) MFMA", "1x1 MFMA GEMM" };
+    return fmt_dup("Conv2d Layer: %d\n Filter dimensions: %dx%d\n Input channels: %d\n Output channels: %d\n"
+                   " Activation: %s\n Stride: %d, %d, %d, %d\n Use bias: %s\n Kernel: %s (variant %d)\n",
+                   node->layerID, c->shape.s0, c->shape.s1, c->shape.s2, c->shape.s3, acts[c->activation & 3],
+                   c->stride.s0, c->stride.s1, c->stride.s2, c->stride.s3, c->useBias ? "Yes" : "No",
+                   algos[c->algo], c->variant);
+}
+
+// ---- schedule: kernel variant and tile parameters for gfx950 -------------------------------------
+gboolean conv_schedule(dR_Graph* net, dR_Node* node) {
+    dR_Conv2d_Data* c = conv_of(node);
+    const int W = c->ishape.s0, H = c->ishape.s1, I = c->shape.s2, O = c->shape.s3;
+    switch (c->algo) {
+        case drConvWinograd: c->variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O); break;
+        case drConv1x1Gemm:  c->variant = drhip_conv1x1_pick_variant(W * H, I, O); break;
+        default:             c->variant = 0; break;      // the direct launcher sizes its own tiles
+    }
+    if ((c->shape.s0 & 1) == 0 || (c->shape.s1 & 1) == 0) {
+        say("Conv2d Layer %d: filter %dx%d must have odd side lengths! \n", node->layerID, c->shape.s0, c->shape.s1);
+        return FALSE;
+    }
+    if (c->activation != tLinear && c->activation != tReLU) {
+        say("Conv2d Layer %d: activation %d is not implemented (0 linear, 1 ReLU)! \n", node->layerID, (int)c->activation);
+        return FALSE;
+    }
+    if (debug(net)) say("Scheduled Conv2D Layer %d: algo %d variant %d\n", node->layerID, (int)c->algo, c->variant);
+    return TRUE;
+}
+
+gboolean conv_create_kernel(dR_Graph*, dR_Node*) { return TRUE; }   // kernels are built into the library
+
+gboolean conv_allocate(dR_Graph* net, dR_Node* node) {
+    dR_Conv2d_Data* c = conv_of(node);
+    const int n = (c->algo == drConvWinograd) ? 16 * c->shape.s2 * c->shape.s3 : weight_count(c);
+    gboolean ok = dR_createFloatBuffer(net, &c->weightsBuf, n, CL_MEM_READ_ONLY);
+    if (c->useBias) ok = ok && dR_createFloatBuffer(net, &c->biasBuf, c->shape.s3, CL_MEM_READ_ONLY);
+    return ok;
+}
+
+gboolean conv_fill(dR_Graph* net, dR_Node* node) {
+    dR_Conv2d_Data* c = conv_of(node);
+    if (!c->hasVariables) { say("Conv2d Layer %d has no weights: call dR_Conv2d_setVariables first! \n", node->layerID); return FALSE; }
+    const size_t rawBytes = (size_t)weight_count(c) * sizeof(float);
+    gboolean ok = TRUE;
+    if (c->algo == drConvWinograd) {
+        // raw weights go up once, U = G g G^T is produced on the device, the raw copy is dropped
+        cl_mem raw = NULL;
+        if (!dR_createFloatBuffer(net, &raw, weight_count(c), CL_MEM_READ_ONLY)) return FALSE;
+        ok = dR_uploadArray(net, (gchar*)"", c->weights, 0, rawBytes, raw);
+        if (ok) ok = !device_failed(net, drhip_winograd_filter_transform_f32((const float*)raw, (float*)c->weightsBuf,
+                                                                              c->shape.s2, c->shape.s3, stream_of(net)),
+                                    "winograd filter transform");
+        if (ok) ok = !device_failed(net, drhip_stream_sync(stream_of(net)), "winograd filter transform (sync)");
+        dR_clMemoryBufferCleanup(net, raw);
+        net->clConfig->memConsumptionGPU -= (glong)rawBytes;
+    } else {
+        ok = dR_uploadArray(net, (gchar*)"", c->weights, 0, rawBytes, c->weightsBuf);
+    }
+    if (ok && c->useBias) ok = dR_uploadArray(net, (gchar*)"", c->biases, 0, (size_t)c->shape.s3 * sizeof(float), c->biasBuf);
+    return ok;
+}
+
+gboolean conv_compute(dR_Graph* net, dR_Node* node) {
+    dR_Conv2d_Data* c = conv_of(node);
+    dR_Node* src = first_input(node);
+    const float* in = dev_out(src);
+    float* out = dev_out(node);
+    const float* w = (const float*)c->weightsBuf;
+    const float* b = c->useBias ? (const float*)c->biasBuf : NULL;
+    const int W = c->ishape.s0, H = c->ishape.s1, I = c->shape.s2, O = c->shape.s3;
+    const int relu = c->activation == tReLU;
+    int rc;
+    switch (c->algo) {
+        case drConvWinograd:
+            rc = drhip_conv3x3_winograd_f32(in, w, b, out, W, H, I, O, relu, c->variant, stream_of(net));
+            break;
+        case drConv1x1Gemm:
+            rc = drhip_conv1x1_f32(in, w, b, out, W * H, I, O, relu, c->variant, stream_of(net));
+            break;
+        default:
+            rc = drhip_conv2d_direct_f32(in, w, b, out, W, H, I, O, c->shape.s0, c->shape.s1,
+                                         c->stride.s1, c->stride.s2, relu, stream_of(net));
+            break;
+    }
+    return !device_failed(net, rc, "deepRACIN:conv2d");
+}
+
+gboolean conv_cleanup_buffers(dR_Graph* net, dR_Node* node) {
+    dR_Conv2d_Data* c = conv_of(node);
+    gboolean ok = dR_clMemoryBufferCleanup(net, c->weightsBuf);
+    if (c->useBias) ok = dR_clMemoryBufferCleanup(net, c->biasBuf) && ok;
+    c->weightsBuf = c->biasBuf = NULL;
+    return ok;
+}
+
+gboolean conv_cleanup_layer(dR_Graph*, dR_Node* node) {
+    dR_Conv2d_Data* c = conv_of(node);
+    if (c->hasVariables) { free(c->weights); if (c->useBias) free(c->biases); }
+    free(c);
+    node->layer = NULL;
+    return TRUE;
+}
+
+}  // namespace
+
+extern "C" {
+
+dR_Node* dR_Conv2d(dR_Graph* net, dR_Node* inputLayer, dR_Shape4* sh, dR_Shape4* st, dR_ActivationType acttype,
+                   gboolean useB) {
+    dR_Conv2d_Data* c = zalloc<dR_Conv2d_Data>();
+    dR_Node* n = zalloc<dR_Node>();
+    c->shape = *sh;
+    c->stride = *st;
+    c->activation = acttype;
+    c->useBias = useB;
+    c->winogradn = 2;
+    n->layer = c;
+    n->type = tConv2d;
+
+    // Same dispatch rule as the reference (src/dR_nodes_conv2d.c:37-81), plus an override for
+    // benchmarking the direct kernel on a layer Winograd would normally take.
+    const bool unitStride = st->s1 == 1 && st->s2 == 1;
+    const char* force = getenv("DR_CONV3X3");
+    if (sh->s0 == 3 && sh->s1 == 3 && unitStride && !(force && strcmp(force, "direct") == 0)) c->algo = drConvWinograd;
+    else if (sh->s0 == 1 && sh->s1 == 1 && unitStride) c->algo = drConv1x1Gemm;
+    else c->algo = drConvDirect;
+
+    n->compute = conv_compute;
+    n->schedule = conv_schedule;
+    n->propagateShape = conv_propagate;
+    n->getRequiredOutputBufferSize = conv_out_size;
+    n->createKernel = conv_create_kernel;
+    n->allocateBuffers = conv_allocate;
+    n->fillBuffers = conv_fill;
+    n->cleanupBuffers = conv_cleanup_buffers;
+    n->cleanupLayer = conv_cleanup_layer;
+    n->printLayer = conv_print;
+    n->serializeNode = conv_serialize;
+    n->parseAppendNode = dR_conv2d_parseAppendNode;
+    n->setVariables = dR_Conv2d_setVariables;
+    n->generateKernel = NULL;
+    n->createKernelName = NULL;
+
+    link_single_input(n, inputLayer, "Conv2d");
+    dR_appendLayer(net, n);
+    return n;
+}
+
+void dR_Conv2d_setVariables(dR_Node* node, gfloat* weights, gfloat* biases) {
+    dR_Conv2d_Data* c = conv_of(node);
+    if (c->hasVariables) { free(c->weights); if (c->useBias) free(c->biases); }
+    c->weights = dup_floats(weights, (size_t)weight_count(c));
+    if (c->useBias) c->biases = dup_floats(biases, (size_t)c->shape.s3);
+    c->hasVariables = TRUE;
+}
+
+dR_Node* dR_conv2d_parseAppendNode(dR_Graph* net, dR_Node** iNodes, gint numINodes, gchar** params, gint numParams,
+                                   gfloat** variables, gint numVariables) {
+    if (numINodes != 1) { say("Parsing Error: Conv2d Node needs 1 InputNodes but got %d!\n", numINodes); return NULL; }
+    if (numParams != 10 || numVariables < 1 || numVariables > 2) {
+        say("Parsing Error: Conv2d Node needs 10 Parameters and 1 or 2 Variables!\n");
+        return NULL;
+    }
+    const int useBias = atoi(params[1]);
+    if (useBias && numVariables < 2) { say("Parsing Error: Conv2d Node uses a bias but has no bias variable!\n"); return NULL; }
+    dR_Shape4 shape = { atoi(params[2]), atoi(params[3]), atoi(params[4]), atoi(params[5]) };
+    dR_Shape4 stride = { atoi(params[6]), atoi(params[7]), atoi(params[8]), atoi(params[9]) };
+    if (!parsed_var_has(0, (size_t)shape.s0 * shape.s1 * shape.s2 * shape.s3, "Conv2d weights")) return NULL;
+    if (useBias && !parsed_var_has(1, (size_t)shape.s3, "Conv2d biases")) return NULL;
+    dR_Node* n = dR_Conv2d(net, iNodes[0], &shape, &stride, (dR_ActivationType)atoi(params[0]), useBias);
+    dR_Conv2d_setVariables(n, variables[0], useBias ? variables[1] : NULL);
+    return n;
+}
+
+}  // extern "C"

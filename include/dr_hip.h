@@ -1,0 +1,158 @@
+/*
+ * dr_hip.h -- the thin C-ABI device layer of the MI355X (gfx950) build of deepRacin.
+ *
+ * This is the layer the host graph code (the dR_* node implementations) calls instead of OpenCL.
+ * It replaces the reference's OpenCL wrapper (src/dR_clwrap.c) and the clSetKernelArg /
+ * clEnqueueNDRangeKernel sequences inside every node's compute() -- plain pointers and sizes only,
+ * no C++ types, no torch types.  All kernels are hand-written HIP for gfx950 and compiled ahead of
+ * time into libdeepracin.so; nothing is generated or compiled at run time.
+ *
+ * Conventions
+ *   - every function returns 0 on success, a negative DRHIP_E* code on failure; a human readable
+ *     message for the calling thread's last failure is available from drhip_last_error();
+ *   - all device pointers are fp32 arrays; tensors are [C][H][W], x fastest (the reference's
+ *     buffer layout, Kernels/dR_helper.cl:15-28);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); launches are
+ *     asynchronous, only drhip_upload / drhip_download / drhip_stream_sync / drhip_event_elapsed_ms
+ *     block;
+ *   - launchers validate shapes on the host and refuse (DRHIP_EINVAL) instead of launching a grid
+ *     that does not match what the kernel assumes.
+ */
+#ifndef DR_HIP_H
+#define DR_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DRHIP_OK         0
+#define DRHIP_EINVAL    -1   /* argument / shape rejected on the host, nothing launched */
+#define DRHIP_EDEVICE   -2   /* a HIP runtime call failed */
+#define DRHIP_ENODEVICE -3   /* no usable gfx950 device */
+
+typedef struct drhip_device_info {
+    char   name[256];
+    char   arch[64];          /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+    int    device;            /* HIP ordinal */
+    int    num_cu;            /* compute units */
+    int    wavefront;         /* 64 on CDNA */
+    int    lds_bytes;         /* max LDS per workgroup */
+    int    clock_khz;
+    size_t hbm_bytes;
+    int    l2_bytes;
+} drhip_device_info;
+
+/* ---- runtime (replaces dR_clInit / dR_clCreateCLContext, reference src/dR_clwrap.c:4-235,592-872) */
+int         drhip_init(int device, drhip_device_info* info /* may be NULL */);
+const char* drhip_last_error(void);
+int         drhip_device_count(void);          /* 0 when no device / no driver; never fails */
+
+/* ---- streams and events (replace the in-order cl_command_queue, src/dR_clwrap.c:90, and the
+ *      cl_event profiling of dR_finishCLKernel, src/dR_clwrap.c:955-1058) */
+int drhip_stream_create(void** stream);
+int drhip_stream_destroy(void* stream);
+int drhip_stream_sync(void* stream);
+int drhip_event_create(void** ev);
+int drhip_event_destroy(void* ev);
+int drhip_event_record(void* ev, void* stream);
+int drhip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms);   /* waits for ev_stop */
+
+/* ---- memory (replace dR_createFloatBuffer :886-899, dR_clMemoryBufferCleanup,
+ *      dR_uploadArray :1079-1143 and dR_downloadArray :1145-1190; both copies block) */
+int drhip_malloc(void** dptr, size_t bytes);
+int drhip_free(void* dptr);
+int drhip_upload(void* dst_dev, size_t dst_byte_offset, const void* src_host, size_t bytes, void* stream);
+int drhip_download(void* dst_host, const void* src_dev, size_t src_byte_offset, size_t bytes, void* stream);
+int drhip_fill_f32(float* dst, float value, size_t n, void* stream);
+
+/* ---- convolution ------------------------------------------------------------------------------
+ * Common meaning: in [I][H][W]; out [O][Ho][Wo] with Wo = W/strideX, Ho = H/strideY (floor);
+ * zero padding of kw/2, kh/2; bias may be NULL; relu != 0 applies max(v,0) after the bias. */
+
+/* Direct correlation, any odd kw x kh and any stride; w is [I][O][kh][kw] exactly as handed to
+ * dR_Conv2d_setVariables.  out[o,y,x] = act(b[o] + sum_{c,j,i} in[c, y*sy+j-kh/2, x*sx+i-kw/2] * w[c][o][j][i]).
+ * Replaces the per-layer generated kernel `conv2d<k>x<k>x<O>_<id>_...` and its launch
+ * (reference src/dR_nodes_conv2d.c:364-420, 481-773); honours the stride as documented at
+ * include/dR_nodes_conv2d.h:47-54. */
+int drhip_conv2d_direct_f32(const float* in, const float* w, const float* bias, float* out,
+                            int W, int H, int I, int O, int kw, int kh,
+                            int strideX, int strideY, int relu, void* stream);
+
+/* Winograd F(2x2,3x3) filter transform U = G g G^T for every (c,o), stored [16][I][O]
+ * (xi = 4*row+col major, o fastest).  Runs once per layer at dR_prepare time.
+ * Replaces the host loop of dR_conv2d_winograd_fillBuffers (src/dR_nodes_conv2d.c:1162-1240);
+ * the reference stores [I][16][O], this build stores xi-major so that each of the 16
+ * transformed-domain GEMMs reads a dense [I][O] panel. */
+int drhip_winograd_filter_transform_f32(const float* w /* [I][O][3][3] */, float* U /* [16][I][O] */,
+                                        int I, int O, void* stream);
+
+/* Fused Winograd F(2x2,3x3) convolution, stride 1, 3x3, SAME zero padding:
+ * input transform B^T d B into LDS, 16 transformed-domain [tiles x I].[I x O] products on the
+ * fp32 MFMA units, output transform A^T m A + bias + ReLU, edge-guarded 2x2 stores.
+ * `variant` selects the tile configuration chosen by the scheduler (0 = let the launcher pick).
+ * Replaces kernel `conv2dwinograd2` and its launch (Kernels/dR_winograd2.cl:23-254,
+ * src/dR_nodes_conv2d.c:1009-1132). */
+int drhip_conv3x3_winograd_f32(const float* in, const float* U, const float* bias, float* out,
+                               int W, int H, int I, int O, int relu, int variant, void* stream);
+/* Tile configuration (variant id >= 1) the gfx950 scheduler assigns to a layer of this shape; the
+ * counterpart of the work-group search in dR_conv2d_winograd_schedule (src/dR_nodes_conv2d.c:809-1006). */
+int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O);
+
+/* 1x1 convolution as an fp32 MFMA GEMM out[O][P] = w[O x I] . in[I][P], P = H*W; w is the
+ * original [I][O] array (no transpose needed).  Replaces kernel `conv2d1x1`, its launch and the
+ * [I][O]->[O][I] re-layout (Kernels/dR_conv2d1x1.cl:4-53, src/dR_nodes_conv2d.c:1605-1716). */
+int drhip_conv1x1_f32(const float* in, const float* w, const float* bias, float* out,
+                      int P, int I, int O, int relu, int variant, void* stream);
+/* Register-tile configuration for a 1x1 layer (replaces dR_conv2d_1x1_schedule, :1526-1602). */
+int drhip_conv1x1_pick_variant(int P, int I, int O);
+
+/* ---- pooling ----------------------------------------------------------------------------------
+ * out dims = ceil(in/stride) per axis; window anchored at (x*stx, y*sty, z*stz); samples outside
+ * the input count as 0.0f; type 0 = max (start value -FLT_MAX), 1 = average (sum / (sx*sy*sz)).
+ * `argmax_out` (may be NULL, max only) receives per output the flat input index of the first
+ * maximum in z,y,x scan order, or -1 if the maximum is a padding zero.
+ * Replaces the generated kernel `Pool<sx>x<sy>_<id>_nocopy{Max,Average}` and its launch
+ * (reference src/dR_nodes_pooling.c:138-183, 277-401). */
+int drhip_pool_f32(const float* in, float* out, int* argmax_out,
+                   int W, int H, int C, int sx, int sy, int sz, int stx, int sty, int stz,
+                   int type, void* stream);
+
+/* ---- fully connected ---------------------------------------------------------------------------
+ * y[n] = act(b[n] + sum_k x[k] * Wt[k][n]), Wt is [K][N] row-major (n fastest), x is the producer's
+ * buffer read linearly.  The reference reads its [C][H][W] input in [H][W][C] order
+ * (Kernels/dR_fcl.cl:78, Kernels/dR_helper.cl:131-142); the host folds that permutation into the
+ * row order of Wt once at prepare time (drhip_fc_permute_rows_f32), so this kernel streams Wt
+ * exactly once, contiguously.  `partials` is scratch of drhip_fc_scratch_floats(K,N) floats
+ * owned by the caller (allocated at prepare time); `counters` is scratch of
+ * drhip_fc_scratch_counters(K,N) ints that must be zero before the first call and is left zero
+ * by every call.  Replaces `matrixVectorMultFirst` + `matrixVectorMultSecond`
+ * (Kernels/dR_fcl.cl:59-120, src/dR_nodes_fc.c:201-278). */
+size_t drhip_fc_scratch_floats(int K, int N);
+size_t drhip_fc_scratch_counters(int K, int N);
+int drhip_fc_f32(const float* x, const float* Wt, const float* bias, float* y,
+                 float* partials, int* counters, int K, int N, int relu, void* stream);
+/* dst[k_chw][n] = src[k_hwc][n] with k_hwc = (y*W + x)*C + z for k_chw = (z*H + y)*W + x. */
+int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, int H, int C, int N, void* stream);
+
+/* ---- softmax: y = exp(x - max x) / sum exp(x - max x) over n elements, one workgroup, wavefront
+ * shuffles.  Replaces computeExp + host-side sum + mulScalar (src/dR_nodes_math.c:620-678,
+ * Kernels/dR_math.cl:216-227,295-305). */
+int drhip_softmax_f32(const float* x, float* y, int n, void* stream);
+
+/* ---- data movement nodes ------------------------------------------------------------------------
+ * copy3d: dst[(z+dz0)][y+dy0][x+dx0] = src[(z+sz0)][y+sy0][x+sx0] for a (w,h,c) box; serves Concat
+ * (generated kernel, src/dR_nodes_transform.c:468-553) and Slice (`extractSlice`,
+ * Kernels/dR_transform.cl:5-24). */
+int drhip_copy3d_f32(const float* src, int sW, int sH, int sx0, int sy0, int sz0,
+                     float* dst, int dW, int dH, int dx0, int dy0, int dz0,
+                     int w, int h, int c, void* stream);
+/* y = f(x, s); op numbering = dR_ElemWise1OperationType: 0 x+s, 1 x-s, 2 x*s, 3 x/s, 4 log x, 5 exp x,
+ * 6 sqrt x, 7 s, 8 pow(x,s)  (`addScalar` ... `powScalar`, Kernels/dR_math.cl:170-341) */
+int drhip_scalar_op_f32(const float* x, float* y, size_t n, int op, float s, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DR_HIP_H */

@@ -1,0 +1,197 @@
+"""End-to-end parity through the deepRacin C graph API (dR_NewGraph ... dR_downloadArray) on the GPU.
+
+Every benchmark configuration is built from seeded synthetic tensors, run through libdeepracin.so and
+compared with the CPU oracle evaluating the same layer list.  Bars (north star): per-layer max
+relative error <= 1e-4 (max|gpu-oracle| / max|oracle| of that layer), final logits max abs error
+<= 1e-3 with identical argmax, pooling bit-exact given equal inputs.
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+import deepracin_amd as dr
+from deepracin_amd import configs
+from conftest import GOLDEN, rel_err
+
+pytestmark = pytest.mark.gpu
+
+LAYER_TOL = 1e-4
+LOGIT_TOL = 1e-3
+
+
+class _Handler(ctypes.Structure):
+    _fields_ = [("outputFor", ctypes.c_void_p), ("size", ctypes.c_int), ("numberOfDependencies", ctypes.c_int),
+                ("bufptr", ctypes.POINTER(ctypes.c_void_p)), ("buf", ctypes.c_void_p)]
+
+
+class _NodeHead(ctypes.Structure):
+    _fields_ = [("oshape", dr.Shape3), ("layerID", ctypes.c_int32), ("previous_layers", ctypes.c_void_p),
+                ("next_layers", ctypes.c_void_p), ("clKernel", ctypes.c_void_p), ("outputBuf", ctypes.POINTER(_Handler))]
+
+
+def node_output(graph, node):
+    """Download a node's buffer via the public struct layout (include/dR_types.h) as [C][H][W]."""
+    head = ctypes.cast(node.ptr, ctypes.POINTER(_NodeHead)).contents
+    s = head.oshape
+    flat = np.empty(s.s0 * s.s1 * s.s2, np.float32)
+    graph.lib.dR_downloadArray(graph.ptr, b"", head.outputBuf.contents.bufptr, 0, flat.nbytes, flat.ctypes.data_as(ctypes.c_void_p))
+    return flat.reshape(s.s2, s.s1, s.s0)
+
+
+def run_config(name, outputs=None, env_vars=None, **kw):
+    spec, feeds, outs = configs.CONFIGS[name](**kw)
+    outs = outputs(spec, outs) if callable(outputs) else (outputs or outs)
+    old = {k: os.environ.get(k) for k in (env_vars or {})}
+    os.environ.update(env_vars or {})
+    try:
+        with dr.Environment() as env:
+            g = env.create_graph()
+            nodes = configs.build_graph(g, spec, outs)
+            dr.prepare(g)
+            for i, a in feeds.items():
+                configs.feed_chw(nodes[i], a)
+            assert g.lib.dR_apply(g.ptr)
+            got = {i: node_output(g, nodes[i]) for i in outs}
+            # a second pass over the same buffers must reproduce the first bit for bit
+            assert g.lib.dR_apply(g.ptr)
+            again = {i: node_output(g, nodes[i]) for i in outs}
+    finally:
+        for k, v in old.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+    for i in outs:
+        assert np.array_equal(got[i], again[i]), "node %d differs between two applies" % i
+    return spec, feeds, got
+
+
+def all_compute_nodes(spec, outs):
+    return [i for i, n in enumerate(spec) if n["op"] != "feed"]
+
+
+def check_layers(oracle, spec, feeds, got, force_direct=False):
+    want = oracle.run_spec(spec, feeds, force_direct=force_direct)
+    for i, g in got.items():
+        assert g.shape == want[i].shape, "node %d shape %s vs %s" % (i, g.shape, want[i].shape)
+        e = rel_err(g, want[i])
+        assert e <= LAYER_TOL, "node %d (%s): rel err %.3g" % (i, spec[i]["op"], e)
+    return want
+
+
+def test_config1_conv3x3_winograd_and_direct(oracle, gpu):
+    spec, feeds, got = run_config("conv3x3")
+    check_layers(oracle, spec, feeds, got)
+    spec, feeds, got_d = run_config("conv3x3", env_vars={"DR_CONV3X3": "direct"})
+    check_layers(oracle, spec, feeds, got_d, force_direct=True)
+    truth = oracle.run_spec(spec, feeds, f64=True)[1]
+    assert rel_err(got[1], truth) <= LAYER_TOL and rel_err(got_d[1], truth) <= LAYER_TOL
+
+
+def test_config2_fire_module(oracle, gpu):
+    # default: only the concat is an output -> producers write straight into the concat buffer
+    spec, feeds, got = run_config("fire")
+    want = check_layers(oracle, spec, feeds, got)
+    assert got[4].shape == (128, 55, 55)
+    # every node an output -> nothing is fused, the concat copies; same numbers
+    spec, feeds, got_all = run_config("fire", outputs=all_compute_nodes)
+    check_layers(oracle, spec, feeds, got_all)
+    assert np.array_equal(got_all[4], got[4])
+    assert np.array_equal(got_all[4][:64], got_all[2]) and np.array_equal(got_all[4][64:], got_all[3])
+    assert rel_err(got[4], oracle.run_spec(spec, feeds, f64=True)[4]) <= LAYER_TOL
+    del want
+
+
+def test_config3_vgg_conv3_block(oracle, gpu):
+    spec, feeds, got = run_config("vgg_conv3", outputs=all_compute_nodes)
+    want = check_layers(oracle, spec, feeds, got)
+    assert got[4].shape == (256, 28, 28)
+    # pooling is bit-exact given the same input: pool the GPU's own conv output on the CPU
+    assert np.array_equal(got[4], oracle.pool(got[3], (2, 2, 1), (2, 2, 1), 0))
+    del want
+
+
+def test_config4_squeezenet(oracle, gpu):
+    spec, feeds, got = run_config("squeezenet", outputs=all_compute_nodes)
+    want = check_layers(oracle, spec, feeds, got)
+    probs, logits = got[len(spec) - 1].reshape(-1), got[len(spec) - 2].reshape(-1)
+    wl = want[len(spec) - 2].reshape(-1)
+    assert np.abs(logits - wl).max() <= LOGIT_TOL
+    assert int(logits.argmax()) == int(wl.argmax()) and int(probs.argmax()) == int(want[-1].argmax())
+    assert abs(float(probs.sum()) - 1) < 1e-4
+    # fused-concat production run gives the same final numbers as the all-outputs run
+    _, _, prod = run_config("squeezenet")
+    assert np.array_equal(prod[len(spec) - 1], got[len(spec) - 1])
+
+
+def test_config5_vgg16(oracle, gpu):
+    spec, feeds, got = run_config("vgg16", outputs=all_compute_nodes)
+    want = check_layers(oracle, spec, feeds, got)
+    logits, wl = got[len(spec) - 2].reshape(-1), want[len(spec) - 2].reshape(-1)
+    assert np.abs(logits - wl).max() <= LOGIT_TOL
+    assert int(logits.argmax()) == int(wl.argmax())
+    probs = got[len(spec) - 1].reshape(-1)
+    assert int(probs.argmax()) == int(want[-1].argmax()) and abs(float(probs.sum()) - 1) < 1e-4
+
+
+@pytest.mark.parametrize("name,cls", [("tiger", 292), ("puzzle", 611)])
+def test_stored_squeezenet_known_answer(oracle, gpu, name, cls):
+    """The reference's only known answers: its stored SqueezeNet v1.1 on its two example images
+    (examples/squeezenet-v1.1/squeezenet_deployed.c:199-207), loaded with dR_loadGraph."""
+    img = np.load(os.path.join(GOLDEN, "%s_224_rgb_u8.npy" % name))
+    chw = np.ascontiguousarray(img.transpose(2, 0, 1).astype(np.float32))
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes, feeds = dr.load_graph(g, os.path.join(GOLDEN, "squeezenet_whole"))
+        assert len(nodes) == 48 and feeds[0].shape == [224, 224, 3]
+        dr.mark_as_output(nodes[-1])
+        dr.mark_as_output(nodes[-2])
+        dr.prepare(g)
+        configs.feed_chw(feeds[0], chw)
+        assert g.lib.dR_apply(g.ptr)
+        probs, pooled = [a.reshape(-1) for a in configs.fetch_chw(g)]
+    want = oracle.run_graph_dir(os.path.join(GOLDEN, "squeezenet_whole"), chw)
+    assert int(probs.argmax()) == cls
+    assert np.abs(pooled - want[-2].reshape(-1)).max() <= LOGIT_TOL
+    assert rel_err(probs, want[-1].reshape(-1)) <= LAYER_TOL
+
+
+def test_python_frontend_hwc_roundtrip(oracle, gpu):
+    """The wrapper's layout rules: HWC in, HWIO weights, HWC out (reference python wrapper :444-497,:559-562)."""
+    rng = np.random.default_rng(3)
+    x = rng.random((10, 12, 5), dtype=np.float32)                     # H, W, C
+    w = (rng.standard_normal((3, 3, 5, 6)) * 0.2).astype(np.float32)  # H, W, I, O
+    b = (rng.standard_normal(6) * 0.1).astype(np.float32)
+    with dr.Environment() as env:
+        g = env.create_graph("HWC")
+        f = dr.feed_node(g, [10, 12, 5])
+        c = dr.Conv2d(f, (3, 3, 5, 6), (1, 1, 1, 1), "relu", w, b)
+        p = dr.Pooling(c, "max", (1, 2, 2, 1), (1, 2, 2, 1))
+        dr.mark_as_output(p)
+        dr.prepare(g)
+        dr.feed_data(f, x)
+        out = dr.apply(g)[0]
+    want = oracle.pool(oracle.conv_winograd(x.transpose(2, 0, 1), w.transpose(2, 3, 0, 1), b, relu=True), (2, 2, 1), (2, 2, 1), 0)
+    assert out.shape == (5, 6, 6)
+    assert rel_err(out, want.transpose(1, 2, 0)) <= LAYER_TOL
+
+
+def test_linearity_at_full_size(gpu):
+    """Size-independent property at VGG scale: a bias-free linear conv commutes with scaling and adds."""
+    rng = np.random.default_rng(5)
+    I, O, S = 128, 256, 56
+    w = (rng.standard_normal((I, O, 3, 3)) * np.sqrt(2.0 / (9 * I))).astype(np.float32)
+    spec = [{"op": "feed", "shape": (S, S, I)}, {"op": "conv", "in": 0, "w": w, "b": None, "stride": (1, 1), "relu": False}]
+    a, b = rng.random((I, S, S), dtype=np.float32), rng.random((I, S, S), dtype=np.float32)
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes = configs.build_graph(g, spec, [1])
+        dr.prepare(g)
+        res = []
+        for inp in (a, b, a + 2 * b):
+            configs.feed_chw(nodes[0], inp)
+            assert g.lib.dR_apply(g.ptr)
+            res.append(configs.fetch_chw(g)[0])
+    assert rel_err(res[2], res[0] + 2 * res[1]) <= LAYER_TOL

@@ -1,0 +1,220 @@
+"""Parity of every hand-written HIP kernel against the CPU oracle, called through the C-ABI
+device layer (include/dr_hip.h) with plain device pointers.
+
+Tolerances (north star): fp32 layers max relative error <= 1e-4, measured as
+max|gpu - oracle| / max|oracle| over the layer; pooling values and max-indices bit-exact.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-4
+RNG = np.random.default_rng(7)
+
+
+def rnd(*shape, scale=1.0):
+    return (RNG.standard_normal(shape) * scale).astype(np.float32)
+
+
+class Dev:
+    """Tiny RAII helper around drhip_malloc/upload/download for the tests."""
+
+    def __init__(self, lib):
+        self.lib = lib
+        self.ptrs = []
+
+    def put(self, arr):
+        arr = np.ascontiguousarray(arr)
+        p = ctypes.c_void_p()
+        assert self.lib.drhip_malloc(ctypes.byref(p), max(arr.nbytes, 4)) == 0, self.lib.drhip_last_error()
+        self.ptrs.append(p)
+        if arr.nbytes:
+            assert self.lib.drhip_upload(p, 0, arr.ctypes.data_as(ctypes.c_void_p), arr.nbytes, None) == 0
+        return p
+
+    def empty(self, n, dtype=np.float32):
+        return self.put(np.full(n, -777, dtype))       # poison: unwritten outputs are visible
+
+    def get(self, p, shape, dtype=np.float32):
+        out = np.empty(shape, dtype)
+        assert self.lib.drhip_download(out.ctypes.data_as(ctypes.c_void_p), p, 0, out.nbytes, None) == 0, self.lib.drhip_last_error()
+        return out
+
+    def close(self):
+        for p in self.ptrs:
+            self.lib.drhip_free(p)
+        self.ptrs = []
+
+
+@pytest.fixture
+def dev(lib, gpu):
+    d = Dev(lib)
+    yield d
+    d.close()
+
+
+def ok(lib, rc):
+    assert rc == 0, lib.drhip_last_error().decode()
+
+
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("W,H,I,O,k,s", [
+    (56, 56, 64, 64, 3, 1),      # config 1, direct variant
+    (224, 224, 3, 64, 3, 2),     # SqueezeNet conv1
+    (17, 13, 5, 7, 3, 1), (20, 18, 4, 20, 5, 1), (33, 31, 3, 9, 3, 2), (16, 16, 2, 3, 7, 3), (9, 9, 1, 1, 1, 2),
+])
+def test_conv_direct(lib, dev, oracle, W, H, I, O, k, s):
+    x, w, b = np.abs(rnd(I, H, W)), rnd(I, O, k, k, scale=np.sqrt(2.0 / (k * k * I))), rnd(O, scale=0.01)
+    want = oracle.conv_direct(x, w, b, (s, s), relu=True)
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_conv2d_direct_f32(dev.put(x), dev.put(w), dev.put(b), out, W, H, I, O, k, k, s, s, 1, None))
+    got = dev.get(out, want.shape)
+    assert rel_err(got, want) <= TOL
+    # linear, no bias
+    want2 = oracle.conv_direct(x, w, None, (s, s), relu=False)
+    ok(lib, lib.drhip_conv2d_direct_f32(dev.put(x), dev.put(w), None, out, W, H, I, O, k, k, s, s, 0, None))
+    assert rel_err(dev.get(out, want2.shape), want2) <= TOL
+
+
+def test_winograd_filter_transform(lib, dev, oracle):
+    I, O = 19, 37
+    w = rnd(I, O, 3, 3)
+    U = dev.empty(16 * I * O)
+    ok(lib, lib.drhip_winograd_filter_transform_f32(dev.put(w), U, I, O, None))
+    got = dev.get(U, (16, I, O))
+    want = oracle.wino_filter(w).transpose(1, 0, 2)      # reference layout [I,16,O] -> xi-major
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+@pytest.mark.parametrize("W,H,I,O", [
+    (56, 56, 64, 64),        # config 1
+    (55, 55, 16, 64),        # fire expand3x3: odd size, I < chunk of 8*2
+    (28, 28, 24, 40),        # I not a multiple of 8, O not a multiple of 32
+    (14, 14, 48, 96), (7, 9, 3, 5), (1, 1, 1, 1), (2, 3, 9, 33), (224, 224, 3, 64),
+])
+def test_winograd_conv(lib, dev, oracle, variant, W, H, I, O):
+    x, w, b = np.abs(rnd(I, H, W)), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
+    U = dev.empty(16 * I * O)
+    ok(lib, lib.drhip_winograd_filter_transform_f32(dev.put(w), U, I, O, None))
+    want = oracle.conv_winograd(x, w, b, relu=True)
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, H, I, O, 1, variant, None))
+    got = dev.get(out, want.shape)
+    assert rel_err(got, want) <= TOL
+    truth = oracle.conv_f64(x, w, b, relu=True)
+    assert rel_err(got, truth) <= TOL
+    # linear, no bias (pre-activation values, sign-sensitive)
+    want2 = oracle.conv_winograd(x, w, None, relu=False)
+    ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, None, out, W, H, I, O, 0, variant, None))
+    assert rel_err(dev.get(out, want2.shape), want2) <= TOL
+
+
+def test_winograd_auto_variant_vgg_shapes(lib, dev, oracle):
+    for (W, I, O) in [(56, 128, 256), (28, 256, 512), (14, 512, 512)]:
+        x, w, b = np.abs(rnd(I, W, W)), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
+        U = dev.empty(16 * I * O)
+        ok(lib, lib.drhip_winograd_filter_transform_f32(dev.put(w), U, I, O, None))
+        want = oracle.conv_winograd(x, w, b, relu=True)
+        out = dev.empty(want.size)
+        ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, W, I, O, 1, 0, None))
+        assert rel_err(dev.get(out, want.shape), want) <= TOL
+        dev.close()
+
+
+def test_winograd_rejects_bad_arguments(lib, dev):
+    p = dev.empty(16)
+    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 0, 4, 1, 1, 0, 0, None) == -1
+    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 4, 4, 1, 1, 0, 9, None) == -1
+    assert lib.drhip_conv3x3_winograd_f32(None, p, None, p, 4, 4, 1, 1, 0, 0, None) == -1
+    assert b"variant" in lib.drhip_last_error() or b"NULL" in lib.drhip_last_error()
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+@pytest.mark.parametrize("P,I,O", [(3025, 128, 16), (3025, 16, 64), (196, 512, 1000), (784, 256, 32), (50, 7, 5), (1, 1, 1), (33, 9, 65)])
+def test_conv1x1(lib, dev, oracle, variant, P, I, O):
+    x, w, b = np.abs(rnd(I, 1, P)), rnd(I, O, 1, 1, scale=np.sqrt(2.0 / I)), rnd(O, scale=0.01)
+    want = oracle.conv1x1(x, w, b, relu=True)
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_conv1x1_f32(dev.put(x), dev.put(w), dev.put(b), out, P, I, O, 1, variant, None))
+    assert rel_err(dev.get(out, want.shape), want) <= TOL
+    want2 = oracle.conv1x1(x, w, None, relu=False)
+    ok(lib, lib.drhip_conv1x1_f32(dev.put(x), dev.put(w), None, out, P, I, O, 0, variant, None))
+    assert rel_err(dev.get(out, want2.shape), want2) <= TOL
+
+
+@pytest.mark.parametrize("W,H,C,k,s", [(56, 56, 256, 2, 2), (112, 112, 64, 3, 2), (55, 55, 7, 3, 2), (14, 14, 1000, 14, 14), (9, 7, 3, 2, 3), (5, 5, 2, 5, 1)])
+def test_pool_bit_exact(lib, dev, oracle, W, H, C, k, s):
+    x = rnd(C, H, W)                     # signed values: the zero padding is observable
+    for kind in (0, 1):
+        want, warg = oracle.pool(x, (k, k, 1), (s, s, 1), kind, want_argmax=True) if kind == 0 else (oracle.pool(x, (k, k, 1), (s, s, 1), kind), None)
+        out = dev.empty(want.size)
+        arg = dev.empty(want.size, np.int32) if kind == 0 else None
+        ok(lib, lib.drhip_pool_f32(dev.put(x), out, arg, W, H, C, k, k, 1, s, s, 1, kind, None))
+        got = dev.get(out, want.shape)
+        if kind == 0:
+            assert np.array_equal(got, want)                                   # values bit-exact
+            assert np.array_equal(dev.get(arg, want.shape, np.int32), warg)    # max-indices bit-exact
+        else:
+            assert rel_err(got, want) <= 1e-6
+
+
+def test_pool_depth_window(lib, dev, oracle):
+    x = rnd(6, 5, 4)
+    want = oracle.pool(x, (2, 2, 2), (2, 2, 2), 0)
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_pool_f32(dev.put(x), out, None, 4, 5, 6, 2, 2, 2, 2, 2, 2, 0, None))
+    assert np.array_equal(dev.get(out, want.shape), want)
+
+
+@pytest.mark.parametrize("C,H,W,N,relu", [(512, 7, 7, 4096, 1), (4096, 1, 1, 1000, 0), (16, 3, 5, 10, 1), (3, 2, 2, 7, 0), (64, 1, 1, 130, 1), (1, 1, 1, 1, 0)])
+def test_fc(lib, dev, oracle, C, H, W, N, relu):
+    K = C * H * W
+    x, Wt, b = np.abs(rnd(C, H, W)), rnd(K, N, scale=np.sqrt(2.0 / K)), rnd(N, scale=0.01)
+    want = oracle.fc(x, Wt, b, relu=bool(relu)).reshape(-1)
+    truth = oracle.fc_f64(x, Wt, b, relu=bool(relu)).reshape(-1)
+    raw, perm = dev.put(Wt), dev.empty(K * N)
+    ok(lib, lib.drhip_fc_permute_rows_f32(raw, perm, W, H, C, N, None))
+    nparts, ncnt = lib.drhip_fc_scratch_floats(K, N), lib.drhip_fc_scratch_counters(K, N)
+    parts, cnt = dev.empty(nparts), dev.put(np.zeros(ncnt, np.int32))
+    y = dev.empty(N)
+    xd, bd = dev.put(x), dev.put(b)
+    for _ in range(2):                     # second call checks that the counters were left at zero
+        ok(lib, lib.drhip_fc_f32(xd, perm, bd, y, parts, cnt, K, N, relu, None))
+        got = dev.get(y, (N,))
+        assert rel_err(got, want) <= TOL and rel_err(got, truth) <= TOL
+    assert np.array_equal(dev.get(cnt, (ncnt,), np.int32), np.zeros(ncnt, np.int32))
+
+
+def test_softmax(lib, dev, oracle):
+    for n, scale in [(1000, 3.0), (10, 1.0), (5000, 5.0), (1, 1.0)]:
+        x = rnd(n, scale=scale)
+        y = dev.empty(n)
+        ok(lib, lib.drhip_softmax_f32(dev.put(x), y, n, None))
+        got = dev.get(y, (n,))
+        assert rel_err(got, oracle.softmax(x)) <= TOL
+        assert rel_err(got, oracle.softmax_f64(x)) <= TOL
+        assert abs(float(got.sum()) - 1) < 1e-5 and int(got.argmax()) == int(x.argmax())
+    # logits that overflow exp() unshifted still give a distribution here
+    big = np.array([100.0, 101.0, 99.0], np.float32)
+    y = dev.empty(3)
+    ok(lib, lib.drhip_softmax_f32(dev.put(big), y, 3, None))
+    assert rel_err(dev.get(y, (3,)), oracle.softmax_f64(big)) <= TOL
+
+
+def test_copy3d_and_scalar(lib, dev, oracle):
+    x = rnd(6, 9, 11)
+    out = dev.empty(3 * 4 * 5)
+    ok(lib, lib.drhip_copy3d_f32(dev.put(x), 11, 9, 2, 3, 1, out, 5, 4, 0, 0, 0, 5, 4, 3, None))
+    assert np.array_equal(dev.get(out, (3, 4, 5)), x[1:4, 3:7, 2:7])
+    assert lib.drhip_copy3d_f32(dev.put(x), 11, 9, 8, 0, 0, out, 5, 4, 0, 0, 0, 5, 4, 3, None) == -1   # box leaves the source
+    for op, s in [(0, 1.5), (1, 123.68), (2, 0.5), (3, 4.0), (7, 2.0)]:
+        y = dev.empty(x.size)
+        ok(lib, lib.drhip_scalar_op_f32(dev.put(x), y, x.size, op, s, None))
+        assert np.array_equal(dev.get(y, x.shape), oracle.scalar_op(x, op, s))
