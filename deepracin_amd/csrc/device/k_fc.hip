@@ -90,7 +90,7 @@ fc_gemv_kernel(const float* __restrict__ x, const float* __restrict__ Wt, const 
                     if (colOk) w[u] = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)(j0 + u) * N));
 #pragma unroll
                 for (int u = 0; u < kFcUnroll; ++u)
-                    if (colOk) fma_row<VEC>(acc, w[u], __builtin_amdgcn_readlane(xl, j0 + u));
+                    if (colOk) fma_row<VEC>(acc, w[u], __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xl), j0 + u)));
             }
         } else {
             for (int j = 0; j < rows; ++j) {
