@@ -1,0 +1,360 @@
+"""Host-side logic of libdeepracin.so that needs no GPU: exported C-ABI, stored-format reader/writer,
+execution order, buffer planner, error behaviour, list cursor rules.  No compute call is made here.
+"""
+import ctypes
+import filecmp
+import os
+import re
+
+import numpy as np
+import pytest
+
+import deepracin_amd as dr
+from deepracin_amd import configs
+from conftest import GOLDEN, ROOT
+
+MODEL = os.path.join(GOLDEN, "squeezenet_whole")
+
+
+# ---------------------------------------------------------------------------------------------
+# C-ABI surface
+# ---------------------------------------------------------------------------------------------
+
+def declared_symbols():
+    names = set()
+    for header in ("deepRACIN.h", "dR_nodes.h", "dr_hip.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        for m in re.finditer(r"\b((?:dR|drhip)_\w+)\s*\(", text):
+            names.add(m.group(1))
+    return sorted(names)
+
+
+def test_library_exports_every_declared_symbol(lib):
+    syms = declared_symbols()
+    assert len(syms) > 60
+    raw = ctypes.CDLL(dr.LIB_PATH)
+    missing = [s for s in syms if not hasattr(raw, s)]
+    assert not missing, "declared in include/*.h but not exported: %s" % missing
+    for must in ("dR_NewGraph", "dR_loadGraph", "dR_feedData", "dR_prepare", "dR_apply", "dR_getOutputBuffers",
+                 "dR_downloadArray", "drhip_conv3x3_winograd_f32", "drhip_conv1x1_f32", "drhip_fc_f32"):
+        assert must in syms
+
+
+def test_no_device_is_reported_not_faked(lib):
+    # on a machine without a GPU the device layer says so; on a GPU box it initialises
+    info = dr.DeviceInfo()
+    rc = lib.drhip_init(0, info)
+    if lib.drhip_device_count() == 0:
+        assert rc == -3 and b"no HIP device" in lib.drhip_last_error()
+    else:
+        assert rc == 0 and info.arch.startswith(b"gfx950")
+
+
+# ---------------------------------------------------------------------------------------------
+# stored format
+# ---------------------------------------------------------------------------------------------
+
+def test_load_stored_model_and_roundtrip_bytes(lib, tmp_path):
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes, feeds = dr.load_graph(g, MODEL)
+        assert len(nodes) == 48 and len(feeds) == 1 and feeds[0].shape == [224, 224, 3]
+        types = [dr.node_struct(n).type for n in nodes]
+        assert types.count(3) == 26 and types.count(16) == 9 and types.count(15) == 3      # conv, concat, slice
+        assert [dr.node_struct(n).layerID for n in nodes] == list(range(48))
+        dr.save_graph(g, str(tmp_path))
+    out = tmp_path / "dr_graph_export"
+    assert filecmp.cmp(str(out / "graph.dr"), os.path.join(MODEL, "graph.dr"), shallow=False)
+    for i in range(52):
+        assert filecmp.cmp(str(out / ("%d.var" % i)), os.path.join(MODEL, "%d.var" % i), shallow=False)
+    # and the written model loads again into the same topology
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes2, _ = dr.load_graph(g, str(out))
+        assert len(nodes2) == 48
+
+
+def test_saved_synthetic_graph_has_reference_grammar(lib, tmp_path):
+    spec, _, outs = configs.fire_module(seed=3, size=9, cin=8, squeeze=4, expand=8)
+    with dr.Environment() as env:
+        g = env.create_graph()
+        configs.build_graph(g, spec, outs)
+        dr.save_graph(g, str(tmp_path))
+    text = open(tmp_path / "dr_graph_export" / "graph.dr").read()
+    lines = text.split("\n")
+    assert lines[0] == "deepRACIN graph: 5 nodes, 1 feed nodes" and text.endswith("\n")
+    assert lines[1:6] == ["Node 0: DataFeedNode", "params: 9 9 8", "previous_nodes:", "next_nodes: 1", "variable_files:"]
+    assert lines[6:11] == ["Node 1: Conv2D", "params: 1 1 1 1 8 4 1 1 1 1", "previous_nodes: 0", "next_nodes: 2 3",
+                           "variable_files: 0.var 1.var"]
+    assert lines[21:26] == ["Node 4: Concat", "params: 2 2", "previous_nodes: 2 3", "next_nodes:", "variable_files:"]
+    w = np.fromfile(tmp_path / "dr_graph_export" / "0.var", dtype="<f4")
+    assert np.array_equal(w, spec[1]["w"].reshape(-1))
+
+
+def _expect_load_failure(tmp_path, text, files=()):
+    d = tmp_path / "m"
+    d.mkdir(exist_ok=True)
+    (d / "graph.dr").write_text(text)
+    for name, arr in files:
+        np.asarray(arr, "<f4").tofile(d / name)
+    with dr.Environment() as env:
+        g = env.create_graph()
+        with pytest.raises(RuntimeError):
+            dr.load_graph(g, str(d))
+
+
+def test_loader_error_paths(lib, tmp_path):
+    feed = "Node 0: DataFeedNode\nparams: 4 4 2\nprevious_nodes:\nnext_nodes: 1\nvariable_files:\n"
+    # missing file
+    with dr.Environment() as env:
+        g = env.create_graph()
+        with pytest.raises(RuntimeError):
+            dr.load_graph(g, str(tmp_path / "nowhere"))
+    # unknown node type
+    _expect_load_failure(tmp_path, "deepRACIN graph: 2 nodes, 1 feed nodes\n" + feed +
+                         "Node 1: Bogus\nparams:\nprevious_nodes: 0\nnext_nodes:\nvariable_files:\n")
+    # node type of the reference that is outside the CNN layer path
+    _expect_load_failure(tmp_path, "deepRACIN graph: 2 nodes, 1 feed nodes\n" + feed +
+                         "Node 1: RGB2Gray\nparams:\nprevious_nodes: 0\nnext_nodes:\nvariable_files:\n")
+    # wrong parameter count for a conv
+    _expect_load_failure(tmp_path, "deepRACIN graph: 2 nodes, 1 feed nodes\n" + feed +
+                         "Node 1: Conv2D\nparams: 1 1 3 3 2\nprevious_nodes: 0\nnext_nodes:\nvariable_files: 0.var 1.var\n",
+                         [("0.var", np.zeros(36)), ("1.var", np.zeros(2))])
+    # variable file shorter than the tensor it should hold
+    _expect_load_failure(tmp_path, "deepRACIN graph: 2 nodes, 1 feed nodes\n" + feed +
+                         "Node 1: Conv2D\nparams: 1 1 3 3 2 2 1 1 1 1\nprevious_nodes: 0\nnext_nodes:\nvariable_files: 0.var 1.var\n",
+                         [("0.var", np.zeros(10)), ("1.var", np.zeros(2))])
+    # forward reference
+    _expect_load_failure(tmp_path, "deepRACIN graph: 2 nodes, 1 feed nodes\n" + feed +
+                         "Node 1: Softmax\nparams:\nprevious_nodes: 1\nnext_nodes:\nvariable_files:\n")
+    # a loader only fills an empty graph
+    with dr.Environment() as env:
+        g = env.create_graph()
+        dr.feed_node(g, [4, 4, 2])
+        with pytest.raises(RuntimeError):
+            dr.load_graph(g, MODEL)
+
+
+# ---------------------------------------------------------------------------------------------
+# prepare-time errors (host side only: fail before any device call)
+# ---------------------------------------------------------------------------------------------
+
+def test_prepare_and_shape_errors(lib):
+    with dr.Environment() as env:
+        g = env.create_graph()
+        assert lib.dR_propagateShapesAndSchedule(g.ptr) == 0            # no feed node
+        mem = (ctypes.c_void_p * 10)()
+        assert lib.dR_getOutputBuffers(g.ptr, mem) == 0                 # not prepared
+        assert lib.dR_apply(g.ptr) == 0
+    rng = np.random.default_rng(0)
+    w = rng.standard_normal((2, 3, 3, 3)).astype(np.float32)
+    with dr.Environment() as env:                                       # conv stride larger than the image -> zero shape
+        g = env.create_graph()
+        spec = [{"op": "feed", "shape": (2, 2, 2)}, {"op": "conv", "in": 0, "w": w, "b": None, "stride": (4, 4), "relu": False}]
+        configs.build_graph(g, spec, [1])
+        assert lib.dR_propagateShapesAndSchedule(g.ptr) == 0
+    with dr.Environment() as env:                                       # FC input size mismatch
+        g = env.create_graph()
+        spec = [{"op": "feed", "shape": (2, 2, 2)}, {"op": "fc", "in": 0, "w": np.zeros((9, 4), np.float32), "b": None, "relu": False}]
+        configs.build_graph(g, spec, [1])
+        assert lib.dR_propagateShapesAndSchedule(g.ptr) == 0
+    with dr.Environment() as env:                                       # conv channel mismatch
+        g = env.create_graph()
+        spec = [{"op": "feed", "shape": (4, 4, 3)}, {"op": "conv", "in": 0, "w": w, "b": None, "stride": (1, 1), "relu": False}]
+        configs.build_graph(g, spec, [1])
+        assert lib.dR_propagateShapesAndSchedule(g.ptr) == 0
+
+
+def test_shape_rules(lib):
+    # conv: floor(in/stride); pool: ceil(in/stride); fc: (N,1,1)   (reference conv2d.c:115, pooling.c:201, fc.c:302)
+    spec, _, outs = configs.squeezenet11(seed=1)
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes = configs.build_graph(g, spec, outs)
+        assert lib.dR_propagateShapesAndSchedule(g.ptr) == 1
+        shapes = [(dr.node_struct(n).oshape.s0, dr.node_struct(n).oshape.s1, dr.node_struct(n).oshape.s2) for n in nodes]
+    _, want = configs.flops(spec)
+    assert shapes == [tuple(s) for s in want]
+    assert shapes[1] == (112, 112, 64) and shapes[2] == (56, 56, 64) and shapes[-1] == (1, 1, 1000)
+    with dr.Environment() as env:
+        g = env.create_graph()
+        spec = [{"op": "feed", "shape": (55, 55, 4)}, {"op": "pool", "in": 0, "window": (3, 3, 1), "stride": (2, 2, 1), "kind": 0}]
+        nodes = configs.build_graph(g, spec, [1])
+        assert lib.dR_propagateShapesAndSchedule(g.ptr) == 1
+        s = dr.node_struct(nodes[1]).oshape
+        assert (s.s0, s.s1, s.s2) == (28, 28, 4)
+
+
+# ---------------------------------------------------------------------------------------------
+# execution order and buffer plan
+# ---------------------------------------------------------------------------------------------
+
+def reference_order(spec):
+    """The reference's work-list walk (src/dR_core.c:121-211) restated over a layer list."""
+    consumers = {i: [] for i in range(len(spec))}
+    inputs = {}
+    for i, n in enumerate(spec):
+        ins = n.get("ins", [n["in"]] if "in" in n else [])
+        inputs[i] = ins
+        for j in ins:
+            consumers[j].append(i)
+    done, queued, work, order = set(), set(), [], []
+    for i, n in enumerate(spec):
+        if n["op"] == "feed":
+            done.add(i)
+            for c in consumers[i]:
+                if c not in queued:
+                    queued.add(c); work.append(c)
+    while work:
+        n = work.pop(0)
+        if not all(j in done for j in inputs[n]):
+            work.append(n)
+            continue
+        done.add(n); order.append(n)
+        for c in consumers[n]:
+            if c not in queued:
+                queued.add(c); work.append(c)
+    return order
+
+
+class FullHandler(ctypes.Structure):
+    pass
+
+
+FullHandler._fields_ = [("outputFor", ctypes.c_void_p), ("size", ctypes.c_int), ("numberOfDependencies", ctypes.c_int),
+                        ("bufptr", ctypes.c_void_p), ("buf", ctypes.c_void_p), ("outputBuf", ctypes.c_int),
+                        ("regionOfInterest", ctypes.c_int), ("useIndexBufferForRoI", ctypes.c_int),
+                        ("indexBuffer", ctypes.c_void_p), ("index", ctypes.c_int), ("roiOrigin", dr.Shape3),
+                        ("drViewOf", ctypes.POINTER(FullHandler)), ("drViewOffset", ctypes.c_int),
+                        ("drFirstDef", ctypes.c_int), ("drLastUse", ctypes.c_int), ("drPinned", ctypes.c_int)]
+
+
+def plan_of(graph, nodes):
+    """[(physical id, offset, size)] per node after dR_planBuffers."""
+    out = []
+    for n in nodes:
+        hp = ctypes.cast(dr.node_struct(n).outputBuf, ctypes.POINTER(FullHandler))
+        h = hp.contents
+        if h.drViewOf:
+            out.append((ctypes.addressof(h.drViewOf.contents), h.drViewOffset, h.size, h.drViewOf.contents.size))
+        else:
+            out.append((ctypes.addressof(h), 0, None, h.size))
+    return out
+
+
+@pytest.mark.parametrize("name", ["fire", "vgg_conv3", "squeezenet", "stored"])
+def test_schedule_order_and_buffer_plan(lib, oracle, name):
+    with dr.Environment() as env:
+        g = env.create_graph()
+        if name == "stored":
+            nodes, _ = dr.load_graph(g, MODEL)
+            spec = oracle.parse_graph_dir(MODEL)
+            outs = [47]
+            dr.mark_as_output(nodes[47])
+        else:
+            kw = {"size": 32} if name == "squeezenet" else {}
+            spec, _, outs = configs.CONFIGS[name](seed=2, **kw)
+            nodes = configs.build_graph(g, spec, outs)
+        assert lib.dR_propagateShapesAndSchedule(g.ptr) == 1
+        pos = [dr.node_struct(n).drSchedulePos for n in nodes]
+        order = [i for _, i in sorted((p, i) for i, p in enumerate(pos) if p >= 0)]
+        assert order == reference_order(spec)
+        assert lib.dR_planBuffers(g.ptr) == 1
+        plan = plan_of(g, nodes)
+        vol = [dr.node_struct(n).oshape.s0 * dr.node_struct(n).oshape.s1 * dr.node_struct(n).oshape.s2 for n in nodes]
+
+    inputs = {i: n.get("ins", [n["in"]] if "in" in n else []) for i, n in enumerate(spec)}
+    last_use = {i: pos[i] for i in range(len(spec))}
+    for i, ins in inputs.items():
+        for j in ins:
+            last_use[j] = max(last_use[j], pos[i])
+    region = {i: (plan[i][0], plan[i][1], plan[i][1] + vol[i]) for i in range(len(spec))}
+    for i in range(len(spec)):
+        assert plan[i][3] >= plan[i][1] + vol[i], "node %d does not fit its buffer" % i
+    fused_into = {}
+    for i, n in enumerate(spec):
+        if n["op"] == "concat" and all(plan[j][0] == plan[i][0] for j in n["ins"]):
+            off = 0
+            for j in n["ins"]:
+                assert plan[j][1] == off, "producer %d not at its channel offset" % j
+                off += vol[j]
+                fused_into[j] = i
+    if name in ("fire", "squeezenet", "stored"):
+        assert fused_into, "channel concats should absorb their producers"
+
+    def overlaps(a, b):
+        return a[0] == b[0] and a[1] < b[2] and b[1] < a[2]
+
+    # brute-force liveness: when node i writes, no other tensor that is still needed may share its bytes
+    for i in range(len(spec)):
+        if pos[i] < 0:
+            continue
+        for j in range(len(spec)):
+            if j == i or fused_into.get(j) == i or fused_into.get(i) == j:
+                continue
+            if j in fused_into and i in fused_into and fused_into[i] == fused_into[j]:
+                assert not overlaps(region[i], region[j])
+                continue
+            live = (pos[j] < pos[i] <= last_use[j]) or spec[j]["op"] == "feed" or j in outs
+            if live and pos[j] <= pos[i]:
+                assert not overlaps(region[i], region[j]), "node %d overwrites live tensor %d" % (i, j)
+    # feed and output tensors own their storage
+    pinned = [i for i, n in enumerate(spec) if n["op"] == "feed"] + list(outs)
+    for i in pinned:
+        assert sum(1 for j in range(len(spec)) if plan[j][0] == plan[i][0] and fused_into.get(j) != i) == 1
+    # and recycling does happen on the deep nets
+    if name in ("squeezenet", "stored"):
+        assert len({p[0] for p in plan}) < len(spec) // 2
+
+
+# ---------------------------------------------------------------------------------------------
+# list cursor rules and helpers
+# ---------------------------------------------------------------------------------------------
+
+def test_list_cursor_rules():
+    raw = ctypes.CDLL(dr.LIB_PATH)
+    vp = ctypes.c_void_p
+    raw.dR_list_createEmptyList.restype = vp
+    raw.dR_list_next.restype = vp
+    raw.dR_list_pop.restype = vp
+    for f in (raw.dR_list_append, raw.dR_list_removeFirstOcc):
+        f.argtypes = [vp, vp]
+    for f in (raw.dR_list_next, raw.dR_list_pop, raw.dR_list_resetIt, raw.dR_list_cleanup):
+        f.argtypes = [vp]
+    l = raw.dR_list_createEmptyList()
+    for v in (11, 22, 33, 44):
+        raw.dR_list_append(l, v)
+    assert [raw.dR_list_next(l) for _ in range(5)] == [11, 22, 33, 44, None]      # wraps to reset after the end
+    assert raw.dR_list_next(l) == 11 and raw.dR_list_next(l) == 22
+    assert raw.dR_list_removeFirstOcc(l, 22) == 1                                  # remove under the cursor
+    assert raw.dR_list_next(l) == 33                                               # successor comes next
+    raw.dR_list_resetIt(l)
+    assert raw.dR_list_next(l) == 11
+    assert raw.dR_list_removeFirstOcc(l, 11) == 1                                  # remove the head under the cursor
+    assert raw.dR_list_next(l) == 33
+    assert raw.dR_list_pop(l) == 33 and raw.dR_list_pop(l) == 44 and raw.dR_list_pop(l) is None
+    assert raw.dR_list_removeFirstOcc(l, 5) == 0
+    raw.dR_list_cleanup(l)
+
+
+def test_matmul_helpers():
+    raw = ctypes.CDLL(dr.LIB_PATH)
+    fp = ctypes.POINTER(ctypes.c_float)
+    rng = np.random.default_rng(1)
+    a, b = rng.standard_normal((4, 3)).astype(np.float32), rng.standard_normal((3, 5)).astype(np.float32)
+    out = np.zeros((4, 5), np.float32)
+    assert raw.dR_matmul(a.ctypes.data_as(fp), 4, 3, b.ctypes.data_as(fp), 3, 5, out.ctypes.data_as(fp)) == 1
+    assert np.allclose(out, a @ b, atol=1e-6)
+    bt = rng.standard_normal((6, 3)).astype(np.float32)
+    out2 = np.zeros((4, 6), np.float32)
+    assert raw.dR_matmulT(a.ctypes.data_as(fp), 4, 3, bt.ctypes.data_as(fp), 6, 3, out2.ctypes.data_as(fp)) == 1
+    assert np.allclose(out2, a @ bt.T, atol=1e-6)
+    assert raw.dR_matmul(a.ctypes.data_as(fp), 4, 3, bt.ctypes.data_as(fp), 6, 3, out2.ctypes.data_as(fp)) == 0
+
+
+def test_pick_variants_are_launchable(lib):
+    for (W, H, I, O) in [(224, 224, 3, 64), (224, 224, 64, 64), (56, 56, 256, 256), (14, 14, 512, 512), (55, 55, 16, 64), (1, 1, 1, 1)]:
+        v = lib.drhip_conv3x3_winograd_pick_variant(W, H, I, O)
+        assert v >= 1
+        assert lib.drhip_conv1x1_pick_variant(W * H, I, O) in (1, 2, 3, 4)
