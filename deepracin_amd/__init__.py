@@ -140,7 +140,9 @@ def load_library(path=None):
         "drhip_event_elapsed_ms": (c_int, [vp, vp, POINTER(c_float)]),
         "drhip_conv2d_direct_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 9 + [vp]),
         "drhip_winograd_filter_transform_f32": (c_int, [vp, vp, c_int, c_int, vp]),
-        "drhip_conv3x3_winograd_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 6 + [vp]),
+        "drhip_conv3x3_winograd_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 6 + [vp, vp]),
+        "drhip_conv3x3_winograd_filter_floats": (c_size_t, [c_int, c_int]),
+        "drhip_conv3x3_winograd_workspace_floats": (c_size_t, [c_int] * 5),
         "drhip_conv3x3_winograd_pick_variant": (c_int, [c_int] * 4),
         "drhip_conv1x1_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 5 + [vp]),
         "drhip_conv1x1_pick_variant": (c_int, [c_int] * 3),

@@ -124,8 +124,17 @@ fc_gemv_kernel(const float* __restrict__ x, const float* __restrict__ Wt, const 
     __threadfence();
     for (int c = tid; c < ncols; c += kFcThreads) {
         const int n = panel * CBW + c;
+        const float* pp = partials + n;
         float s = 0.0f;
-        for (int sl = 0; sl < slices; ++sl) s += __builtin_nontemporal_load(&partials[(size_t)sl * N + n]);
+        int sl = 0;
+        for (; sl + 8 <= slices; sl += 8) {      // 8 independent loads in flight, summed in slice order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = pp[(size_t)(sl + u) * N];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; sl < slices; ++sl) s += pp[(size_t)sl * N];
         if (bias) s += bias[n];
         if (relu) s = fmaxf(s, 0.0f);
         y[n] = s;

@@ -92,9 +92,15 @@ gboolean conv_create_kernel(dR_Graph*, dR_Node*) { return TRUE; }   // kernels a
 
 gboolean conv_allocate(dR_Graph* net, dR_Node* node) {
     dR_Conv2d_Data* c = conv_of(node);
-    const int n = (c->algo == drConvWinograd) ? 16 * c->shape.s2 * c->shape.s3 : weight_count(c);
+    const bool wino = c->algo == drConvWinograd;
+    const int n = wino ? (int)drhip_conv3x3_winograd_filter_floats(c->shape.s2, c->shape.s3) : weight_count(c);
     gboolean ok = dR_createFloatBuffer(net, &c->weightsBuf, n, CL_MEM_READ_ONLY);
     if (c->useBias) ok = ok && dR_createFloatBuffer(net, &c->biasBuf, c->shape.s3, CL_MEM_READ_ONLY);
+    const size_t ws = wino ? drhip_conv3x3_winograd_workspace_floats(c->ishape.s0, c->ishape.s1, c->shape.s2, c->shape.s3, c->variant) : 0;
+    if (ws > 0) {       // split-K partial sums + arrival counters; zeroed once, the kernel keeps the counters at zero
+        ok = ok && dR_createFloatBuffer(net, &c->workspaceBuf, (gint)ws, CL_MEM_READ_WRITE);
+        ok = ok && !device_failed(net, drhip_fill_f32((float*)c->workspaceBuf, 0.0f, ws, stream_of(net)), "conv workspace reset");
+    }
     return ok;
 }
 
@@ -133,7 +139,7 @@ gboolean conv_compute(dR_Graph* net, dR_Node* node) {
     int rc;
     switch (c->algo) {
         case drConvWinograd:
-            rc = drhip_conv3x3_winograd_f32(in, w, b, out, W, H, I, O, relu, c->variant, stream_of(net));
+            rc = drhip_conv3x3_winograd_f32(in, w, b, out, W, H, I, O, relu, c->variant, (float*)c->workspaceBuf, stream_of(net));
             break;
         case drConv1x1Gemm:
             rc = drhip_conv1x1_f32(in, w, b, out, W * H, I, O, relu, c->variant, stream_of(net));
@@ -150,7 +156,8 @@ gboolean conv_cleanup_buffers(dR_Graph* net, dR_Node* node) {
     dR_Conv2d_Data* c = conv_of(node);
     gboolean ok = dR_clMemoryBufferCleanup(net, c->weightsBuf);
     if (c->useBias) ok = dR_clMemoryBufferCleanup(net, c->biasBuf) && ok;
-    c->weightsBuf = c->biasBuf = NULL;
+    ok = dR_clMemoryBufferCleanup(net, c->workspaceBuf) && ok;
+    c->weightsBuf = c->biasBuf = c->workspaceBuf = NULL;
     return ok;
 }
 

@@ -33,7 +33,7 @@ struct dR_Conv2d_Data {
     dR_Shape4           stride;         /* (1, sx, sy, 1) */
     gfloat*             weights;        /* host copy, [I][O][kh][kw] */
     gfloat*             biases;         /* host copy, [O] */
-    cl_mem              weightsBuf;     /* device: direct/1x1 -> [I][O][kh][kw]; Winograd -> U [16][I][O] */
+    cl_mem              weightsBuf;     /* device: direct/1x1 -> [I][O][kh][kw]; Winograd -> transformed filters U */
     cl_mem              biasBuf;
     gboolean            useBias;
     gboolean            hasVariables;
@@ -42,6 +42,7 @@ struct dR_Conv2d_Data {
     dR_ConvAlgo         algo;
     gint                variant;        /* tile configuration id understood by the drhip_* launcher */
     gint                winogradn;      /* always 2: F(2x2,3x3) */
+    cl_mem              workspaceBuf;   /* split-K scratch of the Winograd kernel, NULL when the layer is not split */
 };
 
 /*

@@ -80,25 +80,31 @@ int drhip_conv2d_direct_f32(const float* in, const float* w, const float* bias, 
                             int W, int H, int I, int O, int kw, int kh,
                             int strideX, int strideY, int relu, void* stream);
 
-/* Winograd F(2x2,3x3) filter transform U = G g G^T for every (c,o), stored [16][I][O]
- * (xi = 4*row+col major, o fastest).  Runs once per layer at dR_prepare time.
- * Replaces the host loop of dR_conv2d_winograd_fillBuffers (src/dR_nodes_conv2d.c:1162-1240);
- * the reference stores [I][16][O], this build stores xi-major so that each of the 16
- * transformed-domain GEMMs reads a dense [I][O] panel. */
-int drhip_winograd_filter_transform_f32(const float* w /* [I][O][3][3] */, float* U /* [16][I][O] */,
-                                        int I, int O, void* stream);
+/* Winograd F(2x2,3x3) filter transform U = G g G^T for every (c,o).  Runs once per layer at
+ * dR_prepare time.  U holds drhip_conv3x3_winograd_filter_floats(I,O) floats in the layout the MFMA
+ * kernel streams: U[xi][c/8][o][8] with xi = 4*row+col, input channels padded with zeros to a
+ * multiple of 8, and channel c%8 stored at position (c&1)*4 + (c%8)/2 of its group of 8.
+ * Replaces the host loop of dR_conv2d_winograd_fillBuffers (src/dR_nodes_conv2d.c:1162-1240; the
+ * reference stores [I][16][O]). */
+size_t drhip_conv3x3_winograd_filter_floats(int I, int O);
+int drhip_winograd_filter_transform_f32(const float* w /* [I][O][3][3] */, float* U, int I, int O, void* stream);
 
 /* Fused Winograd F(2x2,3x3) convolution, stride 1, 3x3, SAME zero padding:
  * input transform B^T d B into LDS, 16 transformed-domain [tiles x I].[I x O] products on the
  * fp32 MFMA units, output transform A^T m A + bias + ReLU, edge-guarded 2x2 stores.
- * `variant` selects the tile configuration chosen by the scheduler (0 = let the launcher pick).
- * Replaces kernel `conv2dwinograd2` and its launch (Kernels/dR_winograd2.cl:23-254,
- * src/dR_nodes_conv2d.c:1009-1132). */
+ * `variant` is the configuration chosen by the scheduler: low 4 bits = panel size (1..4), bits 4-7 =
+ * log2 of the number of input-channel splits; 0 lets the launcher pick.  A variant that splits the
+ * input channels needs `workspace` of drhip_conv3x3_winograd_workspace_floats(...) floats, zeroed
+ * once by the caller before the first use (the kernel leaves its counters at zero); otherwise
+ * workspace may be NULL.  Replaces kernel `conv2dwinograd2` and its launch
+ * (Kernels/dR_winograd2.cl:23-254, src/dR_nodes_conv2d.c:1009-1132). */
 int drhip_conv3x3_winograd_f32(const float* in, const float* U, const float* bias, float* out,
-                               int W, int H, int I, int O, int relu, int variant, void* stream);
-/* Tile configuration (variant id >= 1) the gfx950 scheduler assigns to a layer of this shape; the
- * counterpart of the work-group search in dR_conv2d_winograd_schedule (src/dR_nodes_conv2d.c:809-1006). */
+                               int W, int H, int I, int O, int relu, int variant,
+                               float* workspace, void* stream);
+/* Variant id the gfx950 scheduler assigns to a layer of this shape; the counterpart of the
+ * work-group search in dR_conv2d_winograd_schedule (src/dR_nodes_conv2d.c:809-1006). */
 int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O);
+size_t drhip_conv3x3_winograd_workspace_floats(int W, int H, int I, int O, int variant);
 
 /* 1x1 convolution as an fp32 MFMA GEMM out[O][P] = w[O x I] . in[I][P], P = H*W; w is the
  * original [I][O] array (no transpose needed).  Replaces kernel `conv2d1x1`, its launch and the

@@ -82,58 +82,83 @@ def test_conv_direct(lib, dev, oracle, W, H, I, O, k, s):
     assert rel_err(dev.get(out, want2.shape), want2) <= TOL
 
 
+def wino_filters(lib, dev, w):
+    I, O = w.shape[:2]
+    n = lib.drhip_conv3x3_winograd_filter_floats(I, O)
+    U = dev.empty(n)
+    ok(lib, lib.drhip_winograd_filter_transform_f32(dev.put(w), U, I, O, None))
+    return U, n
+
+
+def wino_workspace(lib, dev, W, H, I, O, variant):
+    n = lib.drhip_conv3x3_winograd_workspace_floats(W, H, I, O, variant)
+    return dev.put(np.zeros(n, np.float32)) if n else None
+
+
 def test_winograd_filter_transform(lib, dev, oracle):
     I, O = 19, 37
     w = rnd(I, O, 3, 3)
-    U = dev.empty(16 * I * O)
-    ok(lib, lib.drhip_winograd_filter_transform_f32(dev.put(w), U, I, O, None))
-    got = dev.get(U, (16, I, O))
-    want = oracle.wino_filter(w).transpose(1, 0, 2)      # reference layout [I,16,O] -> xi-major
-    assert np.allclose(got, want, rtol=1e-6, atol=1e-7)
+    U, n = wino_filters(lib, dev, w)
+    chunks = -(-I // 8)
+    assert n == 16 * chunks * 8 * O
+    got = dev.get(U, (16, chunks, O, 8))
+    want = oracle.wino_filter(w)                          # reference layout [I,16,O]
+    # device layout: [xi][c/8][o][pos], channel c%8 at pos (c&1)*4 + (c%8)/2, zero padded
+    expect = np.zeros((16, chunks, O, 8), np.float32)
+    for c in range(I):
+        expect[:, c // 8, :, (c & 1) * 4 + (c % 8) // 2] = want[c]
+    assert np.allclose(got, expect, rtol=1e-6, atol=1e-7)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 0x11, 0x21, 0x12, 0x34])
 @pytest.mark.parametrize("W,H,I,O", [
     (56, 56, 64, 64),        # config 1
-    (55, 55, 16, 64),        # fire expand3x3: odd size, I < chunk of 8*2
+    (55, 55, 16, 64),        # fire expand3x3: odd size, two stages of 8 channels
     (28, 28, 24, 40),        # I not a multiple of 8, O not a multiple of 32
     (14, 14, 48, 96), (7, 9, 3, 5), (1, 1, 1, 1), (2, 3, 9, 33), (224, 224, 3, 64),
 ])
 def test_winograd_conv(lib, dev, oracle, variant, W, H, I, O):
     x, w, b = np.abs(rnd(I, H, W)), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
-    U = dev.empty(16 * I * O)
-    ok(lib, lib.drhip_winograd_filter_transform_f32(dev.put(w), U, I, O, None))
+    U, _ = wino_filters(lib, dev, w)
+    ws = wino_workspace(lib, dev, W, H, I, O, variant)
     want = oracle.conv_winograd(x, w, b, relu=True)
     out = dev.empty(want.size)
-    ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, H, I, O, 1, variant, None))
-    got = dev.get(out, want.shape)
-    assert rel_err(got, want) <= TOL
+    xd, bd = dev.put(x), dev.put(b)
+    for _ in range(2):                       # twice: a split layer must leave its counters at zero
+        ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, out, W, H, I, O, 1, variant, ws, None))
+        got = dev.get(out, want.shape)
+        assert rel_err(got, want) <= TOL
     truth = oracle.conv_f64(x, w, b, relu=True)
     assert rel_err(got, truth) <= TOL
     # linear, no bias (pre-activation values, sign-sensitive)
     want2 = oracle.conv_winograd(x, w, None, relu=False)
-    ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, None, out, W, H, I, O, 0, variant, None))
+    ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, None, out, W, H, I, O, 0, variant, ws, None))
     assert rel_err(dev.get(out, want2.shape), want2) <= TOL
 
 
 def test_winograd_auto_variant_vgg_shapes(lib, dev, oracle):
     for (W, I, O) in [(56, 128, 256), (28, 256, 512), (14, 512, 512)]:
         x, w, b = np.abs(rnd(I, W, W)), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
-        U = dev.empty(16 * I * O)
-        ok(lib, lib.drhip_winograd_filter_transform_f32(dev.put(w), U, I, O, None))
+        U, _ = wino_filters(lib, dev, w)
+        variant = lib.drhip_conv3x3_winograd_pick_variant(W, W, I, O)
+        ws = wino_workspace(lib, dev, W, W, I, O, variant)
         want = oracle.conv_winograd(x, w, b, relu=True)
         out = dev.empty(want.size)
-        ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, W, I, O, 1, 0, None))
+        ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, W, I, O, 1, variant, ws, None))
+        assert rel_err(dev.get(out, want.shape), want) <= TOL
+        # variant 0 without a workspace falls back to an unsplit configuration
+        ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, W, I, O, 1, 0, None, None))
         assert rel_err(dev.get(out, want.shape), want) <= TOL
         dev.close()
 
 
 def test_winograd_rejects_bad_arguments(lib, dev):
-    p = dev.empty(16)
-    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 0, 4, 1, 1, 0, 0, None) == -1
-    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 4, 4, 1, 1, 0, 9, None) == -1
-    assert lib.drhip_conv3x3_winograd_f32(None, p, None, p, 4, 4, 1, 1, 0, 0, None) == -1
-    assert b"variant" in lib.drhip_last_error() or b"NULL" in lib.drhip_last_error()
+    p = dev.empty(64)
+    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 0, 4, 1, 1, 0, 0, None, None) == -1
+    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 4, 4, 1, 1, 0, 9, None, None) == -1
+    assert lib.drhip_conv3x3_winograd_f32(None, p, None, p, 4, 4, 1, 1, 0, 0, None, None) == -1
+    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 4, 4, 32, 1, 0, 0x11, None, None) == -1    # split without workspace
+    assert b"workspace" in lib.drhip_last_error()
 
 
 @pytest.mark.parametrize("variant", [1, 2, 3, 4])
