@@ -97,10 +97,7 @@ gboolean conv_allocate(dR_Graph* net, dR_Node* node) {
     gboolean ok = dR_createFloatBuffer(net, &c->weightsBuf, n, CL_MEM_READ_ONLY);
     if (c->useBias) ok = ok && dR_createFloatBuffer(net, &c->biasBuf, c->shape.s3, CL_MEM_READ_ONLY);
     const size_t ws = wino ? drhip_conv3x3_winograd_workspace_floats(c->ishape.s0, c->ishape.s1, c->shape.s2, c->shape.s3, c->variant) : 0;
-    if (ws > 0) {       // split-K partial sums + arrival counters; zeroed once, the kernel keeps the counters at zero
-        ok = ok && dR_createFloatBuffer(net, &c->workspaceBuf, (gint)ws, CL_MEM_READ_WRITE);
-        ok = ok && !device_failed(net, drhip_fill_f32((float*)c->workspaceBuf, 0.0f, ws, stream_of(net)), "conv workspace reset");
-    }
+    if (ws > 0) ok = ok && dR_createFloatBuffer(net, &c->workspaceBuf, (gint)ws, CL_MEM_READ_WRITE);   // split-K partial tiles
     return ok;
 }
 

@@ -94,8 +94,8 @@ int drhip_winograd_filter_transform_f32(const float* w /* [I][O][3][3] */, float
  * fp32 MFMA units, output transform A^T m A + bias + ReLU, edge-guarded 2x2 stores.
  * `variant` is the configuration chosen by the scheduler: low 4 bits = panel size (1..4), bits 4-7 =
  * log2 of the number of input-channel splits; 0 lets the launcher pick.  A variant that splits the
- * input channels needs `workspace` of drhip_conv3x3_winograd_workspace_floats(...) floats, zeroed
- * once by the caller before the first use (the kernel leaves its counters at zero); otherwise
+ * input channels needs `workspace` of drhip_conv3x3_winograd_workspace_floats(...) floats (scratch,
+ * no initialisation needed; two launches: partial tiles, then their sum in split order); otherwise
  * workspace may be NULL.  Replaces kernel `conv2dwinograd2` and its launch
  * (Kernels/dR_winograd2.cl:23-254, src/dR_nodes_conv2d.c:1009-1132). */
 int drhip_conv3x3_winograd_f32(const float* in, const float* U, const float* bias, float* out,

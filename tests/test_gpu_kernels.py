@@ -99,14 +99,14 @@ def test_winograd_filter_transform(lib, dev, oracle):
     I, O = 19, 37
     w = rnd(I, O, 3, 3)
     U, n = wino_filters(lib, dev, w)
-    chunks = -(-I // 8)
-    assert n == 16 * chunks * 8 * O
-    got = dev.get(U, (16, chunks, O, 8))
+    chunks, opad = -(-I // 8), -(-O // 32) * 32
+    assert n == 16 * chunks * 8 * opad
+    got = dev.get(U, (16, chunks, opad, 8))
     want = oracle.wino_filter(w)                          # reference layout [I,16,O]
-    # device layout: [xi][c/8][o][pos], channel c%8 at pos (c&1)*4 + (c%8)/2, zero padded
-    expect = np.zeros((16, chunks, O, 8), np.float32)
+    # device layout: [xi][c/8][o][pos], channel c%8 at pos (c&1)*4 + (c%8)/2; c and o zero padded
+    expect = np.zeros((16, chunks, opad, 8), np.float32)
     for c in range(I):
-        expect[:, c // 8, :, (c & 1) * 4 + (c % 8) // 2] = want[c]
+        expect[:, c // 8, :O, (c & 1) * 4 + (c % 8) // 2] = want[c]
     assert np.allclose(got, expect, rtol=1e-6, atol=1e-7)
 
 
