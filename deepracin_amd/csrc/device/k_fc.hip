@@ -6,12 +6,13 @@
 //     1 KiB of one row per load instruction (fully coalesced, nontemporal: the matrix is streamed
 //     once and must not evict activations from L2 / Infinity Cache);
 //   - a workgroup (4 waves) owns a panel of CBW = 64*VEC columns and a slice of rows; its waves take
-//     64-row chunks round-robin and keep 8 row loads in flight per lane;
+//     64-row chunks round-robin and keep 8-16 row loads (8-16 KiB per wave) in flight;
 //   - x for a 64-row chunk is loaded once, one element per lane, and broadcast with v_readlane;
 //   - split-K: the grid is (column panels) x (row slices), sized to a few workgroups per CU; each
-//     workgroup writes one partial row, the LAST workgroup of a panel to arrive (device-scope
-//     counter) sums the partials in slice order, adds the bias, applies ReLU and resets the
-//     counter.  Summation order is fixed, so results are reproducible run to run.
+//     workgroup writes one partial row and a second, tiny kernel sums the partials in slice order,
+//     adds the bias and applies ReLU (the same two-step shape as the reference; no device-scope
+//     fences, which on a multi-XCD part cost an L2 write-back per workgroup).  Summation order is
+//     fixed, so results are reproducible run to run.
 //
 // Reference semantics: Kernels/dR_fcl.cl:59-120 (two kernels: partial sums over partitions of K,
 // then a sequential sum of the partials + bias + clamp).  The partition size there depends on the
@@ -56,20 +57,22 @@ static FcPlan fc_plan(int K, int N) {
     return p;
 }
 
+// Partial GEMV of one (column panel, row slice).  slices == 1: writes y directly (bias, ReLU).
+// Otherwise writes partials[slice][n]; fc_reduce_kernel finishes.
 template <int VEC>
 __global__ void __launch_bounds__(kFcThreads)
 fc_gemv_kernel(const float* __restrict__ x, const float* __restrict__ Wt, const float* __restrict__ bias,
-               float* __restrict__ y, float* __restrict__ partials, int* __restrict__ counters,
+               float* __restrict__ y, float* __restrict__ partials,
                int K, int N, int rowsPerSlice, int relu) {
     typedef typename VecT<VEC>::type vec_t;
     constexpr int CBW = kWave * VEC;
     __shared__ float red[kFcWaves][CBW];
-    __shared__ int amLast;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int panel = blockIdx.x, slice = blockIdx.y, slices = gridDim.y;
-    const int col = panel * CBW + lane * VEC;
-    const bool colOk = col < N;                      // N % VEC == 0, so a vector is all-in or all-out
+    // Lanes past the last column re-read the last valid vector (their sums are never stored): the
+    // loads stay unconditional, so the compiler can keep a precise count of loads in flight.
+    const int col = min(panel * CBW + lane * VEC, N - VEC);
     const int rowBegin = slice * rowsPerSlice;
     const int rowEnd = min(K, rowBegin + rowsPerSlice);
 
@@ -79,26 +82,36 @@ fc_gemv_kernel(const float* __restrict__ x, const float* __restrict__ Wt, const 
 
     for (int r0 = rowBegin + wave * kWave; r0 < rowEnd; r0 += kFcWaves * kWave) {
         const int rows = min(kWave, rowEnd - r0);
-        const float xl = (lane < rows) ? x[r0 + lane] : 0.0f;
+        const float xraw = x[min(r0 + lane, K - 1)];
+        const float xl = (lane < rows) ? xraw : 0.0f;
         const float* wp = Wt + (size_t)r0 * N + col;
         if (rows == kWave) {
+            // 64 rows as 8 batches of 8 row loads; two batches (16 KiB per wave) are always in flight
+            vec_t wa[kFcUnroll], wb[kFcUnroll];
 #pragma unroll
-            for (int j0 = 0; j0 < kWave; j0 += kFcUnroll) {
-                vec_t w[kFcUnroll];
+            for (int u = 0; u < kFcUnroll; ++u) wa[u] = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)u * N));
+#pragma unroll
+            for (int j0 = 0; j0 < kWave; j0 += 2 * kFcUnroll) {
 #pragma unroll
                 for (int u = 0; u < kFcUnroll; ++u)
-                    if (colOk) w[u] = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)(j0 + u) * N));
+                    wb[u] = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)(j0 + kFcUnroll + u) * N));
 #pragma unroll
                 for (int u = 0; u < kFcUnroll; ++u)
-                    if (colOk) fma_row<VEC>(acc, w[u], __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xl), j0 + u)));
+                    fma_row<VEC>(acc, wa[u], __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xl), j0 + u)));
+                if (j0 + 2 * kFcUnroll < kWave) {
+#pragma unroll
+                    for (int u = 0; u < kFcUnroll; ++u)
+                        wa[u] = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)(j0 + 2 * kFcUnroll + u) * N));
+                }
+#pragma unroll
+                for (int u = 0; u < kFcUnroll; ++u)
+                    fma_row<VEC>(acc, wb[u], __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xl), j0 + kFcUnroll + u)));
             }
         } else {
             for (int j = 0; j < rows; ++j) {
                 const float xv = __shfl(xl, j, 64);
-                if (colOk) {
-                    vec_t w = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)j * N));
-                    fma_row<VEC>(acc, w, xv);
-                }
+                vec_t w = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)j * N));
+                fma_row<VEC>(acc, w, xv);
             }
         }
     }
@@ -109,37 +122,40 @@ fc_gemv_kernel(const float* __restrict__ x, const float* __restrict__ Wt, const 
     __syncthreads();
     const int ncols = min(CBW, N - panel * CBW);
     for (int c = tid; c < ncols; c += kFcThreads) {
+        const int n = panel * CBW + c;
         float s = red[0][c];
 #pragma unroll
         for (int w = 1; w < kFcWaves; ++w) s += red[w][c];
-        partials[(size_t)slice * N + panel * CBW + c] = s;
-    }
-
-    // last workgroup of this panel finishes the sum
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) amLast = (atomicAdd(&counters[panel], 1) == slices - 1);
-    __syncthreads();
-    if (!amLast) return;
-    __threadfence();
-    for (int c = tid; c < ncols; c += kFcThreads) {
-        const int n = panel * CBW + c;
-        const float* pp = partials + n;
-        float s = 0.0f;
-        int sl = 0;
-        for (; sl + 8 <= slices; sl += 8) {      // 8 independent loads in flight, summed in slice order
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = pp[(size_t)(sl + u) * N];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) s += v[u];
+        if (slices == 1) {
+            if (bias) s += bias[n];
+            if (relu) s = fmaxf(s, 0.0f);
+            y[n] = s;
+        } else {
+            partials[(size_t)slice * N + n] = s;
         }
-        for (; sl < slices; ++sl) s += pp[(size_t)sl * N];
-        if (bias) s += bias[n];
-        if (relu) s = fmaxf(s, 0.0f);
-        y[n] = s;
     }
-    if (tid == 0) counters[panel] = 0;
+}
+
+// y[n] = act(bias[n] + sum over slices of partials[slice][n]), slices added in order.
+__global__ void __launch_bounds__(256)
+fc_reduce_kernel(const float* __restrict__ partials, const float* __restrict__ bias, float* __restrict__ y,
+                 int N, int slices, int relu) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    const float* pp = partials + n;
+    float s = 0.0f;
+    int sl = 0;
+    for (; sl + 8 <= slices; sl += 8) {             // 8 independent loads in flight, summed in slice order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = pp[(size_t)(sl + u) * N];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; sl < slices; ++sl) s += pp[(size_t)sl * N];
+    if (bias) s += bias[n];
+    if (relu) s = fmaxf(s, 0.0f);
+    y[n] = s;
 }
 
 __global__ void __launch_bounds__(256)
@@ -158,30 +174,31 @@ using namespace drhip;
 extern "C" size_t drhip_fc_scratch_floats(int K, int N) {
     if (K <= 0 || N <= 0) return 0;
     FcPlan p = fc_plan(K, N);
-    return (size_t)p.slices * (size_t)N;
-}
-
-extern "C" size_t drhip_fc_scratch_counters(int K, int N) {
-    if (K <= 0 || N <= 0) return 0;
-    return (size_t)fc_plan(K, N).panels;
+    return p.slices > 1 ? (size_t)p.slices * (size_t)N : 0;
 }
 
 extern "C" int drhip_fc_f32(const float* x, const float* Wt, const float* bias, float* y,
-                            float* partials, int* counters, int K, int N, int relu, void* stream) {
-    DRHIP_REQUIRE(x && Wt && y && partials && counters, "drhip_fc_f32: NULL pointer");
+                            float* partials, int K, int N, int relu, void* stream) {
+    DRHIP_REQUIRE(x && Wt && y, "drhip_fc_f32: NULL pointer");
     DRHIP_REQUIRE(K > 0 && N > 0, "drhip_fc_f32: bad shape K=%d N=%d", K, N);
     FcPlan p = fc_plan(K, N);
+    DRHIP_REQUIRE(p.slices == 1 || partials, "drhip_fc_f32: this shape is split over %d row slices and needs the partials scratch", p.slices);
     DRHIP_REQUIRE(((size_t)Wt % (4 * p.vec)) == 0, "drhip_fc_f32: weight matrix not aligned for %d-wide loads", p.vec);
     DRHIP_REQUIRE(p.slices <= 65535, "drhip_fc_f32: too many row slices");
     dim3 grid(p.panels, p.slices), block(kFcThreads);
     hipStream_t s = as_stream(stream);
     if (p.vec == 4)
-        hipLaunchKernelGGL((fc_gemv_kernel<4>), grid, block, 0, s, x, Wt, bias, y, partials, counters, K, N, p.rowsPerSlice, relu);
+        hipLaunchKernelGGL((fc_gemv_kernel<4>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
     else if (p.vec == 2)
-        hipLaunchKernelGGL((fc_gemv_kernel<2>), grid, block, 0, s, x, Wt, bias, y, partials, counters, K, N, p.rowsPerSlice, relu);
+        hipLaunchKernelGGL((fc_gemv_kernel<2>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
     else
-        hipLaunchKernelGGL((fc_gemv_kernel<1>), grid, block, 0, s, x, Wt, bias, y, partials, counters, K, N, p.rowsPerSlice, relu);
-    return launched("fc_gemv_kernel");
+        hipLaunchKernelGGL((fc_gemv_kernel<1>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
+    if (int rc = launched("fc_gemv_kernel")) return rc;
+    if (p.slices > 1) {
+        hipLaunchKernelGGL(fc_reduce_kernel, dim3(ceil_div(N, 256)), dim3(256), 0, s, partials, bias, y, N, p.slices, relu);
+        return launched("fc_reduce_kernel");
+    }
+    return DRHIP_OK;
 }
 
 extern "C" int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, int H, int C, int N, void* stream) {

@@ -114,8 +114,8 @@ gboolean fc_allocate(dR_Graph* net, dR_Node* node) {
     if ((long long)K * N >= (1ll << 31)) { say("FullyConnected Layer %d: %dx%d weights exceed 2^31 elements! \n", node->layerID, K, N); return FALSE; }
     gboolean ok = dR_createFloatBuffer(net, &f->weightsBuf, K * N, CL_MEM_READ_ONLY);
     if (f->useBias) ok = ok && dR_createFloatBuffer(net, &f->biasBuf, N, CL_MEM_READ_ONLY);
-    ok = ok && dR_createFloatBuffer(net, &f->partialsBuf, (gint)drhip_fc_scratch_floats(K, N), CL_MEM_READ_WRITE);
-    ok = ok && dR_createFloatBuffer(net, &f->countersBuf, (gint)drhip_fc_scratch_counters(K, N), CL_MEM_READ_WRITE);
+    const size_t scratch = drhip_fc_scratch_floats(K, N);
+    if (scratch > 0) ok = ok && dR_createFloatBuffer(net, &f->partialsBuf, (gint)scratch, CL_MEM_READ_WRITE);
     return ok;
 }
 
@@ -141,15 +141,13 @@ gboolean fc_fill(dR_Graph* net, dR_Node* node) {
         net->clConfig->memConsumptionGPU -= (glong)bytes;
     }
     if (ok && f->useBias) ok = dR_uploadArray(net, (gchar*)"", f->biases, 0, (size_t)N * sizeof(float), f->biasBuf);
-    if (ok) ok = !device_failed(net, drhip_fill_f32((float*)f->countersBuf, 0.0f, drhip_fc_scratch_counters(K, N), stream_of(net)),
-                                "fc counter reset");
     return ok;
 }
 
 gboolean fc_compute(dR_Graph* net, dR_Node* node) {
     dR_FC_Data* f = fc_of(node);
     int rc = drhip_fc_f32(dev_out(first_input(node)), (const float*)f->weightsBuf, f->useBias ? (const float*)f->biasBuf : NULL,
-                          dev_out(node), (float*)f->partialsBuf, (int*)f->countersBuf, f->shape.s0, f->shape.s1,
+                          dev_out(node), (float*)f->partialsBuf, f->shape.s0, f->shape.s1,
                           f->activation == tReLU, stream_of(net));
     return !device_failed(net, rc, "deepRACIN:FullyConnected");
 }
@@ -159,8 +157,7 @@ gboolean fc_cleanup_buffers(dR_Graph* net, dR_Node* node) {
     gboolean ok = dR_clMemoryBufferCleanup(net, f->weightsBuf);
     if (f->useBias) ok = dR_clMemoryBufferCleanup(net, f->biasBuf) && ok;
     ok = dR_clMemoryBufferCleanup(net, f->partialsBuf) && ok;
-    ok = dR_clMemoryBufferCleanup(net, f->countersBuf) && ok;
-    f->weightsBuf = f->biasBuf = f->partialsBuf = f->countersBuf = NULL;
+    f->weightsBuf = f->biasBuf = f->partialsBuf = NULL;
     return ok;
 }
 

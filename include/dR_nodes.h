@@ -92,8 +92,7 @@ struct dR_FC_Data {
     gboolean            hasVariables;
     dR_ActivationType   activation;
     /* gfx950 plan */
-    cl_mem              partialsBuf;    /* split-K partial sums */
-    cl_mem              countersBuf;    /* arrival counters of the last-block reduction */
+    cl_mem              partialsBuf;    /* split-K partial sums, NULL when the layer is not split */
 };
 
 /* y[n] = act(b[n] + sum_k x_hwc[k] * W[k][n]); shape = (K, N); K must equal W*H*C of the input. */

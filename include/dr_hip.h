@@ -130,15 +130,14 @@ int drhip_pool_f32(const float* in, float* out, int* argmax_out,
  * buffer read linearly.  The reference reads its [C][H][W] input in [H][W][C] order
  * (Kernels/dR_fcl.cl:78, Kernels/dR_helper.cl:131-142); the host folds that permutation into the
  * row order of Wt once at prepare time (drhip_fc_permute_rows_f32), so this kernel streams Wt
- * exactly once, contiguously.  `partials` is scratch of drhip_fc_scratch_floats(K,N) floats
- * owned by the caller (allocated at prepare time); `counters` is scratch of
- * drhip_fc_scratch_counters(K,N) ints that must be zero before the first call and is left zero
- * by every call.  Replaces `matrixVectorMultFirst` + `matrixVectorMultSecond`
+ * exactly once, contiguously.  `partials` is scratch of drhip_fc_scratch_floats(K,N) floats owned by
+ * the caller (allocated at prepare time, no initialisation needed): the row range is split over
+ * workgroups and a second small kernel sums the partial rows in fixed order (0 floats = the shape is
+ * not split and partials may be NULL).  Replaces `matrixVectorMultFirst` + `matrixVectorMultSecond`
  * (Kernels/dR_fcl.cl:59-120, src/dR_nodes_fc.c:201-278). */
 size_t drhip_fc_scratch_floats(int K, int N);
-size_t drhip_fc_scratch_counters(int K, int N);
 int drhip_fc_f32(const float* x, const float* Wt, const float* bias, float* y,
-                 float* partials, int* counters, int K, int N, int relu, void* stream);
+                 float* partials, int K, int N, int relu, void* stream);
 /* dst[k_chw][n] = src[k_hwc][n] with k_hwc = (y*W + x)*C + z for k_chw = (z*H + y)*W + x. */
 int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, int H, int C, int N, void* stream);
 
