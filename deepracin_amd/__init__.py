@@ -129,6 +129,10 @@ def load_library(path=None):
         "drhip_last_error": (c_char_p, []),
         "drhip_device_count": (c_int, []),
         "drhip_stream_sync": (c_int, [vp]),
+        "drhip_graph_capture_begin": (c_int, [vp]),
+        "drhip_graph_capture_end": (c_int, [vp, POINTER(vp)]),
+        "drhip_graph_launch": (c_int, [vp, vp]),
+        "drhip_graph_destroy": (c_int, [vp]),
         "drhip_malloc": (c_int, [POINTER(vp), c_size_t]),
         "drhip_free": (c_int, [vp]),
         "drhip_upload": (c_int, [vp, c_size_t, vp, c_size_t, vp]),

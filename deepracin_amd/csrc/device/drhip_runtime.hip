@@ -87,6 +87,41 @@ int drhip_event_elapsed_ms(void* a, void* b, float* ms) {
     return check(hipEventElapsedTime(ms, (hipEvent_t)a, (hipEvent_t)b), "hipEventElapsedTime");
 }
 
+int drhip_graph_capture_begin(void* stream) {
+    DRHIP_REQUIRE(stream, "drhip_graph_capture_begin: the default stream cannot be captured");
+    return check(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+}
+
+int drhip_graph_capture_end(void* stream, void** graph_exec) {
+    DRHIP_REQUIRE(stream && graph_exec, "drhip_graph_capture_end: NULL argument");
+    *graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    hipError_t e = hipStreamEndCapture(as_stream(stream), &graph);
+    if (e != hipSuccess || !graph) {
+        (void)hipGetLastError();
+        if (graph) (void)hipGraphDestroy(graph);
+        return fail(DRHIP_EDEVICE, "hipStreamEndCapture: %s", hipGetErrorString(e));
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(DRHIP_EDEVICE, "hipGraphInstantiate: %s", hipGetErrorString(e));
+    }
+    *graph_exec = (void*)exec;
+    return DRHIP_OK;
+}
+
+int drhip_graph_launch(void* graph_exec, void* stream) {
+    DRHIP_REQUIRE(graph_exec, "drhip_graph_launch: NULL graph");
+    return check(hipGraphLaunch((hipGraphExec_t)graph_exec, as_stream(stream)), "hipGraphLaunch");
+}
+
+int drhip_graph_destroy(void* graph_exec) {
+    return graph_exec ? check(hipGraphExecDestroy((hipGraphExec_t)graph_exec), "hipGraphExecDestroy") : DRHIP_OK;
+}
+
 int drhip_malloc(void** dptr, size_t bytes) {
     DRHIP_REQUIRE(dptr && bytes > 0, "drhip_malloc: NULL out-pointer or zero size");
     return check(hipMalloc(dptr, bytes), "hipMalloc");

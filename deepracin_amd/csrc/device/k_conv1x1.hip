@@ -2,8 +2,8 @@
 //
 //   out[o][p] = act(b[o] + sum_c w[c][o] * in[c][p]),   p = y*W + x,  P = H*W
 //
-// MFMA-bound in principle (2*P*I*O FLOP; bytes 4*(P*I + I*O + O + P*O)), in practice the
-// SqueezeNet layers are a few MFLOP each and the launch dominates.
+// MFMA-bound in principle (2*P*I*O FLOP; bytes 4*(P*I + I*O + O + P*O)); the SqueezeNet layers are
+// a few MFLOP each, so what matters is latency: enough waves, loads kept in flight, no second launch.
 //
 // Both operands are already laid out the way v_mfma_f32_32x32x2_f32 wants them:
 //   A (32 rows x 2 k): lane -> (row = lane%32, k = lane/32).  rows = output channels, and the
@@ -12,10 +12,15 @@
 //     fillBuffers (src/dR_nodes_conv2d.c:1696-1716) is not needed;
 //   B (2 k x 32 cols): lane -> (col = lane%32, k = lane/32).  cols = pixels, in[c][p] is
 //     contiguous in p;
-//   D: lane -> col (pixel) lane%32, register r -> row (channel) 8*(r/4) + 4*(lane/32) + r%4, so
-//     every store instruction writes 2 x 128 contiguous bytes of two output-channel rows.
-// No LDS: each wave owns a (32*WM channels) x (32*WN pixels) tile and streams its operands from
-// L2 with a register prefetch of the next 8 input channels.
+//   D: lane -> col (pixel) lane%32, register r -> row (channel) 8*(r/4) + 4*(lane/32) + r%4.
+//
+// One workgroup = one 32-channel x 32-pixel output tile, KW waves (1, 2, 4 or 8).  The input channels
+// are dealt to the waves in stages of 8 (wave w takes stages w, w+KW, ...); every wave streams its
+// operands straight from L2 with the next two stages already in flight (loads are unconditional
+// from clamped addresses, zero padding is a select afterwards, so the compiler can count them),
+// and the KW partial tiles are added in wave order through LDS before bias, ReLU and a coalesced
+// store.  Splitting the channel loop inside the workgroup gives the 14x14 layers (7 pixel tiles)
+// enough waves without a second kernel or atomics, and keeps the summation order fixed.
 //
 // Reference kernel: Kernels/dR_conv2d1x1.cl:4-53 (one work-item per (x,y,o), sequential sum over
 // the input channels).
@@ -25,108 +30,100 @@ namespace drhip {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int kC1Threads = 256;
-constexpr int kC1KC = 8;            // channels per prefetch group (4 MFMA k-steps)
+constexpr int kC1KC = 8;            // channels per stage (4 MFMA k-steps)
+constexpr int kC1Pad = 33;          // LDS row pitch of a partial tile (floats)
 
-template <int WM, int WN>
-__global__ void __launch_bounds__(kC1Threads)
+__global__ void __launch_bounds__(512)
 conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
-                    float* __restrict__ out, int P, int I, int O, int nPT, int nTiles, int relu) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+                    float* __restrict__ out, int P, int I, int O, int nPT, int relu) {
+    extern __shared__ float part[];                 // [KW][32][kC1Pad], used only when KW > 1
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int KW = blockDim.x >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
-    const int tile = blockIdx.x * (kC1Threads / kWave) + wave;      // one tile per wave
-    if (tile >= nTiles) return;
-    const int o0 = (tile / nPT) * 32 * WM;
-    const int p0 = (tile % nPT) * 32 * WN;
+    const int o0 = (blockIdx.x / nPT) * 32, p0 = (blockIdx.x % nPT) * 32;
+    const int nStages = (I + kC1KC - 1) / kC1KC;
 
-    f32x16 acc[WM][WN];
+    f32x16 acc;
 #pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-        for (int j = 0; j < WN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
 
-    float aCur[kC1KC / 2][WM], bCur[kC1KC / 2][WN], aNxt[kC1KC / 2][WM], bNxt[kC1KC / 2][WN];
-    auto load_group = [&](float (&a)[kC1KC / 2][WM], float (&b)[kC1KC / 2][WN], int c0) {
+    // clamped operand columns: always valid addresses; out-of-range lanes are zeroed by select
+    const int oL = min(o0 + l32, O - 1), pL = min(p0 + l32, P - 1);
+    const bool oOk = o0 + l32 < O, pOk = p0 + l32 < P;
+    float aA[4], bA[4], aB[4], bB[4];
+    auto load_stage = [&](float (&a)[4], float (&b)[4], int stage) {
+        stage = min(stage, nStages - 1);
 #pragma unroll
-        for (int ks = 0; ks < kC1KC / 2; ++ks) {
-            const int c = c0 + 2 * ks + lhi;
-#pragma unroll
-            for (int i = 0; i < WM; ++i) {
-                const int o = o0 + 32 * i + l32;
-                a[ks][i] = (c < I && o < O) ? w[(size_t)c * O + o] : 0.0f;
-            }
-#pragma unroll
-            for (int j = 0; j < WN; ++j) {
-                const int p = p0 + 32 * j + l32;
-                b[ks][j] = (c < I && p < P) ? in[(size_t)c * P + p] : 0.0f;
-            }
+        for (int ks = 0; ks < 4; ++ks) {
+            const int c = min(stage * kC1KC + 2 * ks + lhi, I - 1);
+            a[ks] = w[(size_t)c * O + oL];
+            b[ks] = in[(size_t)c * P + pL];
         }
     };
-
-    const int nGroups = (I + kC1KC - 1) / kC1KC;
-    load_group(aCur, bCur, 0);
-    for (int gI = 0; gI < nGroups; ++gI) {
-        const bool more = gI + 1 < nGroups;
-        if (more) load_group(aNxt, bNxt, (gI + 1) * kC1KC);
+    auto multiply = [&](const float (&a)[4], const float (&b)[4], int stage) {
 #pragma unroll
-        for (int ks = 0; ks < kC1KC / 2; ++ks)
-#pragma unroll
-            for (int i = 0; i < WM; ++i)
-#pragma unroll
-                for (int j = 0; j < WN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(aCur[ks][i], bCur[ks][j], acc[i][j], 0, 0, 0);
-        if (more) {
-#pragma unroll
-            for (int ks = 0; ks < kC1KC / 2; ++ks) {
-#pragma unroll
-                for (int i = 0; i < WM; ++i) aCur[ks][i] = aNxt[ks][i];
-#pragma unroll
-                for (int j = 0; j < WN; ++j) bCur[ks][j] = bNxt[ks][j];
-            }
+        for (int ks = 0; ks < 4; ++ks) {
+            const bool cOk = stage * kC1KC + 2 * ks + lhi < I;
+            const float av = (cOk && oOk) ? a[ks] : 0.0f;
+            const float bv = (cOk && pOk) ? b[ks] : 0.0f;
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
         }
+    };
+    // stages wave, wave+KW, ...; two in flight
+    int st = wave;
+    load_stage(aA, bA, st);
+    load_stage(aB, bB, st + KW);
+    for (; st + KW < nStages; st += 2 * KW) {
+        multiply(aA, bA, st);
+        load_stage(aA, bA, st + 2 * KW);
+        multiply(aB, bB, st + KW);
+        load_stage(aB, bB, st + 3 * KW);
     }
+    if (st < nStages) multiply(aA, bA, st);
 
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
+    if (KW == 1) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int o = o0 + 32 * i + 8 * (r / 4) + 4 * lhi + (r % 4);
-            if (o >= O) continue;
-            const float bv = bias ? bias[o] : 0.0f;
-#pragma unroll
-            for (int j = 0; j < WN; ++j) {
-                const int p = p0 + 32 * j + l32;
-                if (p >= P) continue;
-                float v = acc[i][j][r] + bv;
+            const int o = o0 + 8 * (r / 4) + 4 * lhi + (r % 4);
+            if (o < O && pOk) {
+                float v = acc[r] + (bias ? bias[o] : 0.0f);
                 if (relu) v = fmaxf(v, 0.0f);
-                out[(size_t)o * P + p] = v;
+                out[(size_t)o * P + p0 + l32] = v;
             }
         }
-}
-
-template <int WM, int WN>
-static int launch_c1(const float* in, const float* w, const float* bias, float* out, int P, int I, int O, int relu, hipStream_t s) {
-    const int nPT = ceil_div(P, 32 * WN), nOT = ceil_div(O, 32 * WM), nTiles = nPT * nOT;
-    const int blocks = ceil_div(nTiles, kC1Threads / kWave);
-    hipLaunchKernelGGL((conv1x1_mfma_kernel<WM, WN>), dim3(blocks), dim3(kC1Threads), 0, s, in, w, bias, out, P, I, O, nPT, nTiles, relu);
-    return launched("conv1x1_mfma_kernel");
+        return;
+    }
+    // partial tiles -> LDS, then all lanes add them in wave order
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        part[(wave * 32 + 8 * (r / 4) + 4 * lhi + (r % 4)) * kC1Pad + l32] = acc[r];
+    __syncthreads();
+    for (int idx = tid; idx < 32 * 32; idx += blockDim.x) {
+        const int ol = idx >> 5, pl = idx & 31;
+        const int o = o0 + ol, p = p0 + pl;
+        float s = 0.0f;
+        for (int k = 0; k < KW; ++k) s += part[(k * 32 + ol) * kC1Pad + pl];
+        if (o < O && p < P) {
+            if (bias) s += bias[o];
+            if (relu) s = fmaxf(s, 0.0f);
+            out[(size_t)o * P + p] = s;
+        }
+    }
 }
 
 }  // namespace drhip
 
 using namespace drhip;
 
-// Register tile per wave: as large as still leaves one wave per SIMD something to do.
+// Waves per output tile: as many as give every wave at least two 8-channel stages, more when the
+// layer has few tiles.  variant = number of waves (1, 2, 4, 8).
 extern "C" int drhip_conv1x1_pick_variant(int P, int I, int O) {
-    (void)I;
-    const int simds = 4 * num_cu();
-    auto tiles = [&](int wm, int wn) { return ceil_div(O, 32 * wm) * ceil_div(P, 32 * wn); };
-    if (O > 32 && P > 32 && tiles(2, 2) >= simds) return 4;
-    if (P > 32 && tiles(1, 2) >= simds) return 3;
-    if (O > 32 && tiles(2, 1) >= simds) return 2;
-    return 1;
+    const int tiles = ceil_div(O, 32) * ceil_div(P, 32);
+    const int stages = ceil_div(I, kC1KC);
+    int kw = 1;
+    while (kw < 8 && stages >= 4 * kw && tiles * kw < 8 * num_cu()) kw *= 2;
+    return kw;
 }
 
 extern "C" int drhip_conv1x1_f32(const float* in, const float* w, const float* bias, float* out,
@@ -136,12 +133,10 @@ extern "C" int drhip_conv1x1_f32(const float* in, const float* w, const float* b
     DRHIP_REQUIRE((long long)P * I < (1ll << 31) && (long long)P * O < (1ll << 31) && (long long)I * O < (1ll << 31),
                   "drhip_conv1x1_f32: tensor too large for 32-bit indexing");
     if (variant == 0) variant = drhip_conv1x1_pick_variant(P, I, O);
-    hipStream_t s = as_stream(stream);
-    switch (variant) {
-        case 1: return launch_c1<1, 1>(in, w, bias, out, P, I, O, relu, s);
-        case 2: return launch_c1<2, 1>(in, w, bias, out, P, I, O, relu, s);
-        case 3: return launch_c1<1, 2>(in, w, bias, out, P, I, O, relu, s);
-        case 4: return launch_c1<2, 2>(in, w, bias, out, P, I, O, relu, s);
-        default: return fail(DRHIP_EINVAL, "drhip_conv1x1_f32: unknown variant %d", variant);
-    }
+    DRHIP_REQUIRE(variant == 1 || variant == 2 || variant == 4 || variant == 8, "drhip_conv1x1_f32: unknown variant %d (waves per tile: 1, 2, 4, 8)", variant);
+    const int nPT = ceil_div(P, 32), nOT = ceil_div(O, 32);
+    const size_t ldsBytes = variant > 1 ? (size_t)variant * 32 * kC1Pad * sizeof(float) : 0;
+    hipLaunchKernelGGL(conv1x1_mfma_kernel, dim3(nPT * nOT), dim3(64 * variant), ldsBytes, as_stream(stream),
+                       in, w, bias, out, P, I, O, nPT, relu);
+    return launched("conv1x1_mfma_kernel");
 }

@@ -139,7 +139,10 @@ void dR_feedData(dR_Graph* net, dR_Node* feednode, gfloat* data, gint offset, gi
 }
 
 // One forward pass: walks the schedule and lets every node enqueue its kernels.  Asynchronous
-// unless profiling is enabled (reference src/deepRACIN.c:204-270: clFlush only).
+// unless profiling is enabled (reference src/deepRACIN.c:204-270: clFlush only).  The first plain
+// pass records the node walk into a hipGraph; later passes replay it with a single launch.
+// DR_HIPGRAPH=0 in the environment, profilingGPU, a debug layer, or a node whose compute() cannot
+// be captured (it blocks or allocates) keep the node-by-node path.
 //
 // profilingGPU: the reference waits for every kernel and reads its cl_event (src/dR_clwrap.c:970-1049).
 // Here one hipEvent is recorded between consecutive nodes while the whole pass is enqueued without
@@ -155,6 +158,43 @@ gboolean dR_apply(dR_Graph* net) {
 
     std::chrono::steady_clock::time_point t0;
     if (profCPU) { t0 = std::chrono::steady_clock::now(); net->config->totalNodeCPUTime = 0.0; }
+
+    // Plain passes are replayed from a hipGraph captured on the first one: at batch 1 the nodes are
+    // so short that enqueueing them one by one costs more host time than they take to run.
+    if (!profGPU && net->debugLayer < 0 && !net->drGraphOff) {
+        if (!net->drGraphExec) {
+            const char* env = getenv("DR_HIPGRAPH");
+            if ((env && strcmp(env, "0") == 0) || drhip_graph_capture_begin(cc->hipStream) != DRHIP_OK) {
+                net->drGraphOff = TRUE;
+            } else {
+                bool recorded = true;
+                for (dR_ListElement* e = net->scheduledLayers->first; e && recorded; e = e->next) {
+                    dR_Node* node = (dR_Node*)e->element;
+                    recorded = node->compute(net, node);
+                }
+                void* exec = NULL;
+                const int rc = drhip_graph_capture_end(cc->hipStream, &exec);
+                if (!recorded || rc != DRHIP_OK) {
+                    if (exec) drhip_graph_destroy(exec);
+                    net->drGraphOff = TRUE;         // a node that cannot be captured: enqueue node by node from now on
+                    if (debug(net)) say("dR_apply: forward pass not capturable, running node by node\n");
+                } else {
+                    net->drGraphExec = exec;
+                }
+            }
+        }
+        if (net->drGraphExec) {
+            if (device_failed(net, drhip_graph_launch(net->drGraphExec, cc->hipStream), "dR_apply(graph)")) return FALSE;
+            if (profCPU) {
+                if (device_failed(net, drhip_stream_sync(cc->hipStream), "dR_apply(sync)")) return FALSE;
+                double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+                net->drLastApplyMs = ms;
+                say("CPU Profiling: Whole graph took: %2.3fms, Sum of all nodes: %2.3fms \n", ms, net->config->totalNodeCPUTime);
+            }
+            if (net->config->debugInfo) say("Done.\n\n");
+            return TRUE;
+        }
+    }
 
     const int nNodes = net->scheduledLayers->length;
     if (profGPU && cc->hipNumEvents < nNodes + 1) {
@@ -208,6 +248,7 @@ void dR_cleanup(dR_Graph* net, gboolean cleanupcl) {
     const bool talk = verbose(net);
     if (talk) say("Cleaning up deepRACIN...\n");
     if (net->clConfig->clContext) drhip_stream_sync(net->clConfig->hipStream);
+    if (net->drGraphExec) { drhip_graph_destroy(net->drGraphExec); net->drGraphExec = NULL; }
     if (net->prepared) dR_cleanupBuffers(net);
     if (cleanupcl) dR_cleanupCL(net);
     dR_cleanupNet(net);

@@ -181,6 +181,8 @@ struct dR_Graph {
     /* ---- additions of this build ---- */
     dR_List*        drViewHandlers;         /* handlers that alias a slice of a stream buffer */
     gdouble         drLastApplyMs;          /* wall ms of the last dR_apply when profilingCPU */
+    void*           drGraphExec;            /* hipGraphExec_t of the captured forward pass, NULL until captured */
+    gboolean        drGraphOff;             /* TRUE: always enqueue node by node (capture failed or DR_HIPGRAPH=0) */
 };
 
 struct dR_MemoryHandler {

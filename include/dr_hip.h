@@ -59,6 +59,16 @@ int drhip_event_destroy(void* ev);
 int drhip_event_record(void* ev, void* stream);
 int drhip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms);   /* waits for ev_stop */
 
+/* ---- launch graphs: record everything enqueued on `stream` between begin and end into an executable
+ *      hipGraph and replay it with one call.  Used by dR_apply to take the per-node launch cost
+ *      (dozens of small kernels at batch 1) off the host.  capture_end returns DRHIP_EDEVICE and a NULL
+ *      graph if something that cannot be captured (a blocking call, an allocation) happened in
+ *      between; the stream is usable again afterwards. */
+int drhip_graph_capture_begin(void* stream);
+int drhip_graph_capture_end(void* stream, void** graph_exec);
+int drhip_graph_launch(void* graph_exec, void* stream);
+int drhip_graph_destroy(void* graph_exec);
+
 /* ---- memory (replace dR_createFloatBuffer :886-899, dR_clMemoryBufferCleanup,
  *      dR_uploadArray :1079-1143 and dR_downloadArray :1145-1190; both copies block) */
 int drhip_malloc(void** dptr, size_t bytes);

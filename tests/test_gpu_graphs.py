@@ -195,3 +195,52 @@ def test_linearity_at_full_size(gpu):
             assert g.lib.dR_apply(g.ptr)
             res.append(configs.fetch_chw(g)[0])
     assert rel_err(res[2], res[0] + 2 * res[1]) <= LAYER_TOL
+
+
+def _run_many(spec, outs, inputs, graph_mode):
+    old = os.environ.get("DR_HIPGRAPH")
+    os.environ["DR_HIPGRAPH"] = "1" if graph_mode else "0"
+    try:
+        with dr.Environment() as env:
+            g = env.create_graph()
+            nodes = configs.build_graph(g, spec, outs)
+            dr.prepare(g)
+            res = []
+            for x in inputs:
+                configs.feed_chw(nodes[0], x)          # eager blocking copy between the replays
+                assert g.lib.dR_apply(g.ptr)
+                res.append([a.copy() for a in configs.fetch_chw(g)])   # blocking download = sync
+            used_graph = bool(ctypes.cast(g.ptr, ctypes.POINTER(_GraphTail)).contents.drGraphExec)
+    finally:
+        if old is None:
+            os.environ.pop("DR_HIPGRAPH", None)
+        else:
+            os.environ["DR_HIPGRAPH"] = old
+    return res, used_graph
+
+
+class _GraphTail(ctypes.Structure):
+    """dR_Graph (include/dR_types.h) up to the launch-graph fields."""
+    _fields_ = [("prepared", ctypes.c_int), ("swapBuffer1", ctypes.c_void_p), ("swapBuffer2", ctypes.c_void_p),
+                ("config", ctypes.c_void_p), ("clConfig", ctypes.c_void_p), ("feed_layers", ctypes.c_void_p),
+                ("output_layers", ctypes.c_void_p), ("streamBufferHandlers", ctypes.c_void_p),
+                ("number_of_layers", ctypes.c_int32), ("maxBufferSize", ctypes.c_int32), ("hostDebugBuffer", ctypes.c_void_p),
+                ("scheduledLayers", ctypes.c_void_p), ("allNodes", ctypes.c_void_p), ("debugLayer", ctypes.c_int),
+                ("drViewHandlers", ctypes.c_void_p), ("drLastApplyMs", ctypes.c_double), ("drGraphExec", ctypes.c_void_p),
+                ("drGraphOff", ctypes.c_int)]
+
+
+@pytest.mark.parametrize("name", ["squeezenet", "vgg_conv3"])
+def test_launch_graph_replays_equal_node_by_node(gpu, name):
+    """dR_apply replays a captured hipGraph after the first pass.  Every replay -- with blocking copies
+    and synchronisations of the program in between -- must equal the node-by-node result bit for bit."""
+    spec, feeds, outs = configs.CONFIGS[name](seed=9)
+    rng = np.random.default_rng(10)
+    inputs = [feeds[0]] + [rng.random(feeds[0].shape, dtype=np.float32) for _ in range(4)] + [feeds[0]]
+    eager, g0 = _run_many(spec, outs, inputs, graph_mode=False)
+    replay, g1 = _run_many(spec, outs, inputs, graph_mode=True)
+    assert not g0 and g1, "graph mode flags: eager run used a graph=%s, graph run used a graph=%s" % (g0, g1)
+    for k, (a, b) in enumerate(zip(eager, replay)):
+        for x, y in zip(a, b):
+            assert np.array_equal(x, y), "replay %d differs from the node-by-node pass" % k
+    assert np.array_equal(replay[0][0], replay[-1][0])

@@ -161,8 +161,8 @@ def test_winograd_rejects_bad_arguments(lib, dev):
     assert b"workspace" in lib.drhip_last_error()
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4])
-@pytest.mark.parametrize("P,I,O", [(3025, 128, 16), (3025, 16, 64), (196, 512, 1000), (784, 256, 32), (50, 7, 5), (1, 1, 1), (33, 9, 65)])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8])
+@pytest.mark.parametrize("P,I,O", [(3025, 128, 16), (3025, 16, 64), (196, 512, 1000), (196, 512, 64), (784, 256, 32), (50, 7, 5), (1, 1, 1), (33, 9, 65), (70, 24, 40)])
 def test_conv1x1(lib, dev, oracle, variant, P, I, O):
     x, w, b = np.abs(rnd(I, 1, P)), rnd(I, O, 1, 1, scale=np.sqrt(2.0 / I)), rnd(O, scale=0.01)
     want = oracle.conv1x1(x, w, b, relu=True)
