@@ -15,33 +15,24 @@
 //   M_xi[o][t] = sum_c U_xi[c][o] * V_xi[c][t]        (t = 2x2 tile index)
 //
 // and run on the fp32 matrix cores (v_mfma_f32_32x32x2_f32, 64 FLOP/clk/SIMD, MFMA-bound:
-// algorithmic work 2*9*H*W*I*O FLOP direct-equivalent, 2*16*tiles*I*O FLOP issued).
-//
-// A workgroup owns TB = 32*MT tiles x OB = 32*NT output channels for all 16 xi and consumes the
-// input channels 8 at a time ("stage"):
-//   1. a producer lane loads the 4x4 input window of one (tile, channel) pair straight from global
-//      memory (zero padded by predication) two stages ahead of its use;
-//   2. B^T d B in registers (32 adds), result written to LDS as V[xi][c][t]  (double buffered);
-//   3. per k-step of 2 channels a consumer wave issues MFMAs with A = U_xi[c][o] (read from global
-//      memory, where dR_prepare stored it so that the four k-steps of a stage are one 16-byte load
-//      per lane and 1 KiB contiguous per wave) and B = V_xi[c][t] (one conflict-free ds_read_b32);
-//   4. epilogue: accumulators go through LDS 16 output channels at a time so that one lane sees
-//      all 16 xi of one (tile, o), applies A^T m A, bias, ReLU and stores the 2x2 pixels
-//      (adjacent lanes = adjacent tiles, 8-byte stores, edge guarded for odd sizes).
+// algorithmic work 2*9*H*W*I*O FLOP direct-equivalent, 2*16*tiles*I*O FLOP issued).  The input
+// transform happens in registers, the output transform in registers and LDS; see the kernel.
 // Workgroup ids are remapped so that each XCD (own L2) works on a contiguous range of
 // output-channel panels and therefore touches only its share of U.
-// Layers with few tiles (28x28, 14x14) cannot fill 256 CUs with panels alone: there the input
-// channels are split over gridDim.y workgroups whose partial outputs are summed, in fixed order,
-// by a small second kernel (deterministic, no float atomics, no device-scope fences).
+// Layers with few tiles cannot fill 256 CUs with panels alone: there the input channels are split
+// over gridDim.y workgroups whose partial outputs are summed, in fixed order, by a small second
+// kernel (deterministic, no float atomics, no device-scope fences).
 #include "drhip_common.hpp"
+
+#include <type_traits>
 
 namespace drhip {
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kWinoThreads = 512;
-constexpr int kWinoKC = 8;          // input channels per LDS stage
+constexpr int kWinoThreads = 256;       // 4 waves, one per row of the 4x4 transform
+constexpr int kWinoKC = 8;          // input channels per stage (4 MFMA k-steps)
 constexpr int kXcds = 8;            // L2 domains of MI355X
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -92,26 +83,6 @@ winograd_filter_transform_kernel(const float* __restrict__ w, float* __restrict_
     for (int k = 0; k < 16; ++k) U[wino_u_index(k, c, o, nChunks, Opad)] = u[k];
 }
 
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also fences global memory, which
-// on gfx9 means s_waitcnt vmcnt(0): every global load issued for a later stage would have to land
-// before the barrier and the software pipeline would collapse.  Nothing in this kernel passes data
-// between lanes through global memory, so the LDS-only form is sufficient.
-__device__ inline void wino_lds_barrier() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-// Output transform of one (tile, o): right factor A first, then A^T (order of the reference kernel).
-__device__ inline void wino_output_transform(const float (&m)[16], float& y00, float& y01, float& y10, float& y11) {
-    const float s0 = m[0] + m[1] + m[2],    s1 = m[1] - m[2] + m[3];
-    const float s2 = m[4] + m[5] + m[6],    s3 = m[5] - m[6] + m[7];
-    const float s4 = m[8] + m[9] + m[10],   s5 = m[9] - m[10] + m[11];
-    const float s6 = m[12] + m[13] + m[14], s7 = m[13] - m[14] + m[15];
-    y00 = s0 + s2 + s4; y01 = s1 + s3 + s5;
-    y10 = s2 - s4 + s6; y11 = s3 - s5 + s7;
-}
-
 // 2x2 store with edge guards; vec2: W even and the base 8-byte aligned.
 __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, int vec2,
                                        float y00, float y01, float y10, float y11) {
@@ -129,35 +100,54 @@ __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, 
     }
 }
 
-// Workgroup = 512 lanes = 8 waves, split by role (a CU places wave i on SIMD i%4, so every SIMD
-// hosts one wave of each role and interleaves their instructions):
-//   waves 0-3  "consumers": wave w owns xi = 4w..4w+3 of the panel; they only read operands and
-//              issue MFMAs (A = transformed filters from global memory, prefetched two stages
-//              ahead; B = V from LDS);
-//   waves 4-7  "producers": load the 4x4 input windows (two stages ahead, in registers), apply
-//              B^T d B and write V[xi][c][t] into the LDS buffer the consumers will read next.
-// One barrier per 8-channel stage keeps the two roles in lock step; V is double buffered, so the
-// producers fill stage s+1 while the consumers multiply stage s.  The two roles run separate loops
-// behind a wave-uniform (scalar) branch and execute the same number of barriers; keeping their
-// code apart lets each loop wait only for its own loads and lets the registers of one role be
-// reused by the other.
+// One wavefront per row of the 4x4 transform.
+//
+// On gfx950 an fp32 MFMA and an fp32 VALU instruction never overlap on one SIMD (measured: a wave
+// issuing MFMAs and a second wave issuing FMAs on the same SIMD take the sum of their times), so
+// every VALU instruction in the channel loop is paid for in matrix throughput.  The loop is therefore
+// built to need almost none:
+//
+//   * wave w (0..3) of a 256-lane workgroup owns the transform positions xi = 4w..4w+3, i.e. row w
+//     of B^T d B.  That row needs only TWO rows of the 4x4 input window (row w combined with row 2
+//     or 1), so a lane loads 8 floats and spends 8 adds per (tile, channel) - and the four results
+//     are exactly the B operands (lane -> tile lane%32, k -> channel parity lane/32) of that wave's
+//     own MFMAs.  V never goes through LDS and the waves of a workgroup never synchronise inside
+//     the channel loop.
+//   * the window samples are fetched with raw buffer loads whose resource covers the channels from
+//     the current one to the end of the tensor: samples outside the image carry an offset beyond
+//     the resource, channels past the last one see a resource of size zero, and the hardware
+//     returns 0.0 for both - zero padding and ragged channel counts cost no instruction.
+//   * all addresses are a per-lane byte offset computed once plus scalar (SGPR) bases.
+//   * operands of the next stage are loaded into the registers the current stage has just
+//     finished with (input rows after their transform, filters after the MFMAs of their xi pair),
+//     so every load has one full stage to land.
+// A workgroup owns 32 tiles x OB = 32*NT output channels; the larger OB, the more MFMAs share the
+// 8 adds of a transformed input sample.  Epilogue: each wave applies the right factor A to its row
+// (in registers), the four rows meet in LDS (32 KiB) and every lane finishes A^T . for its
+// (tile, channel) pairs, adds bias, applies ReLU and stores 2x2 pixels (adjacent lanes = adjacent
+// tiles).
 //
 // gridDim.y = number of input-channel splits KS.  KS == 1: the workgroup finishes its outputs.
 // KS > 1: every split stores its partial (pre-bias) 2x2 tiles, tile-major, to the workspace and
 // winograd_split_reduce_kernel sums them in split order, adds the bias and applies ReLU.
-template <int MT, int NT>
-__global__ void __launch_bounds__(kWinoThreads)
+constexpr unsigned kBufferFlags = 0x00020000u;      // dword 3 of a gfx9 raw buffer resource (32-bit data format)
+constexpr unsigned kOutOfRange = 0x80000000u;       // byte offset no resource of at most 2 GiB contains
+
+__device__ inline float buf_load(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)voffset, (int)soffset, 0));
+}
+__device__ inline f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset) {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voffset, (int)soffset, 0));
+}
+
+template <int NT>
+__global__ void __launch_bounds__(kWinoThreads, (NT == 1 ? 3 : (NT == 2 ? 2 : 1)))
 winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__ U,
                          const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
                          int W, int H, int I, int O, int tilesX, int T, int nTB, int nBlocks,
                          int chunksPerSplit, int relu, int vec2) {
-    constexpr int TB = 32 * MT, OB = 32 * NT, KC = kWinoKC;
-    constexpr int PT = kWinoThreads / 2;            // lanes per role (256)
-    constexpr int CSTEP = PT / TB;                  // channel distance between a producer lane's pairs
-    constexpr int PAIRS = TB * KC / PT;             // (tile, channel) pairs per producer lane and stage (= MT)
-    constexpr int VSZ = 16 * KC * TB;               // floats per V buffer
-    constexpr int OSTEP = kWinoThreads / TB;        // output channels covered by one sweep of all lanes
-    extern __shared__ float lds[];                  // 2 * VSZ floats
+    constexpr int TB = 32, OB = 32 * NT, KC = kWinoKC;
+    extern __shared__ float P[];                    // epilogue only: [4 rows][2][OB o][32 t] floats
 
     // ---- which panel: XCD-aware remap of the linear workgroup id -----------------------------
     const int perXcd = gridDim.x / kXcds;           // grid is padded to a multiple of kXcds
@@ -168,220 +158,168 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     const int split = blockIdx.y, nSplits = gridDim.y;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // scalar: the role branch is uniform
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // = row of the transform
     const int l32 = lane & 31, lhi = lane >> 5;
-    const size_t plane = (size_t)H * W;
+    const int plane = H * W;
     const int nChunksAll = (I + KC - 1) / KC;
     const int chBegin = split * chunksPerSplit;
     const int chEnd = min(nChunksAll, chBegin + chunksPerSplit);    // > chBegin: the launcher creates no empty split
     const int Opad = wino_opad(O);
-    float* const V0 = lds;
-    float* const V1 = lds + VSZ;
 
-    auto tile_xy = [&](int tLocal, int& txo, int& tyo) {
-        const int tg = t0 + tLocal;
-        const bool okT = tg < T;
-        tyo = okT ? tg / tilesX : 0;
-        txo = okT ? tg % tilesX : 0;
-        return okT;
+    // ---- this lane's tile and the byte offsets of the two window rows it reads ---------------
+    // Row w of B^T d:  w=0: d0 - d2,  w=1: d1 + d2,  w=2: d2 - d1,  w=3: d3 - d1.
+    const int tg = t0 + l32;
+    const bool tileOk = tg < T;
+    const int ty = tileOk ? tg / tilesX : 0, tx = tileOk ? tg % tilesX : 0;
+    const int x0 = 2 * tx - 1, y0 = 2 * ty - 1;
+    const int rowA = wave, rowB = (wave < 2) ? 2 : 1;
+    const float sgn = (wave == 1) ? 1.0f : -1.0f;
+    unsigned offA[4], offB[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        const int x = x0 + s, ya = y0 + rowA, yb = y0 + rowB;
+        const bool xOk = tileOk && x >= 0 && x < W;
+        offA[s] = (xOk && ya >= 0 && ya < H) ? 4u * (unsigned)(lhi * plane + ya * W + x) : kOutOfRange;
+        offB[s] = (xOk && yb >= 0 && yb < H) ? 4u * (unsigned)(lhi * plane + yb * W + x) : kOutOfRange;
+    }
+    // Window rows of channels cbase + lhi.  "Ranged" form: the resource starts at channel cbase and
+    // ends with the tensor, so channels >= I read 0 without touching memory (ragged last chunk,
+    // prefetch past the end).  "Plain" form for chunks known to lie inside the tensor: one resource
+    // for the whole tensor, the channel offset travels in the scalar offset (a resource that changes
+    // inside the loop makes the compiler wait for all outstanding loads at the loop head).
+    const __amdgpu_buffer_rsrc_t rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kBufferFlags);
+    auto load_rows_plain = [&](float (&d)[8], int cbase) {
+        const unsigned soff = 4u * (unsigned)(cbase * plane);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { d[s] = buf_load(rIn, offA[s], soff); d[4 + s] = buf_load(rIn, offB[s], soff); }
+    };
+    auto load_rows_ranged = [&](float (&d)[8], int cbase) {
+        const int left = max(I - cbase, 0);
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(in + (size_t)min(cbase, I) * plane), 0,
+                                                                             left * plane * 4, kBufferFlags);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { d[s] = buf_load(r, offA[s], 0); d[4 + s] = buf_load(r, offB[s], 0); }
+    };
+    // filters of one xi for a whole stage: component ks of the 16-byte load = k-step ks
+    const __amdgpu_buffer_rsrc_t rU = __builtin_amdgcn_make_buffer_rsrc((void*)U, 0, 16 * nChunksAll * Opad * 8 * 4, kBufferFlags);
+    const unsigned fOff = 4u * (unsigned)((o0 + l32) * 8 + 4 * lhi);
+    auto load_filters = [&](f32x4 (&f)[NT], int e, int chunk) {
+        const unsigned soff = 4u * (unsigned)(((4 * wave + e) * nChunksAll + chunk) * Opad * 8);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) f[nt] = buf_load4(rU, fOff + 4u * (unsigned)(nt * 32 * 8), soff);
     };
 
-    // ---- epilogue helper (all 512 lanes): read the 16 xi of one (tile, o) from LDS, transform, store
-    float* Ms = lds;                                // [16 xi][16 o][TB t]  == 2 * VSZ floats
-    const bool direct = nSplits == 1;
-    const int et = tid % TB;                        // this lane's tile in the epilogue
-    const int eo = tid / TB;                        // this lane's first channel within a 16-channel pass
-    int etx, ety;
-    const bool eTileOk = tile_xy(et, etx, ety);
-    const int ox = 2 * etx, oy = 2 * ety;
-    f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
-    auto emit_pass = [&](int nt, int h) {
+    f32x16 acc[4][NT];
 #pragma unroll
-        for (int q = 0; q < 16 / OSTEP; ++q) {
-            const int oo = eo + q * OSTEP;          // 0..15
-            const int ol = 32 * nt + 16 * h + oo;
-            const int o = o0 + ol;
-            float m[16];
+    for (int e = 0; e < 4; ++e)
 #pragma unroll
-            for (int xi = 0; xi < 16; ++xi) m[xi] = Ms[(xi * 16 + oo) * TB + et];
-            float y00, y01, y10, y11;
-            wino_output_transform(m, y00, y01, y10, y11);
-            if (direct) {
-                if (eTileOk && o < O) {
-                    if (bias) { const float bv = bias[o]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
-                    if (relu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
-                    wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, y00, y01, y10, y11);
-                }
-            } else {
-                f32x4 v = {y00, y01, y10, y11};
-                wsTiles[(size_t)ol * TB + et] = v;  // whole panel, padding included: 1 KiB per wave
-            }
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[e][nt][r] = 0.0f;
+
+    float raw[4][8];
+    f32x4 f[4][NT];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) load_rows_ranged(raw[ks], chBegin * KC + 2 * ks);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) load_filters(f[e], e, chBegin);
+
+    // One stage: transform the rows of chunk ch (and start loading those of chunk ch+1 into the
+    // same registers), then 16*NT MFMAs, reloading the filters of each xi pair behind its MFMAs.
+    auto stage = [&](int ch, auto plainNext) {
+        const int next = min(ch + 1, nChunksAll - 1);
+        float b[4][4];                              // [k-step][xi within the row]
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            float m[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) m[s] = fmaf(sgn, raw[ks][4 + s], raw[ks][s]);   // exact: sgn is +-1
+            b[ks][0] = m[0] - m[2];
+            b[ks][1] = m[1] + m[2];
+            b[ks][2] = m[2] - m[1];
+            b[ks][3] = m[3] - m[1];
         }
-    };
-
-    if (wave < 4) {
-        // =================================== consumers ===========================================
-        f32x16 acc[4][NT][MT];
+        __builtin_amdgcn_sched_barrier(0);
+        // 8 slots of 2*NT MFMAs (two xi at a time: dependent MFMAs stay 2*NT apart).  The loads of
+        // the next stage are issued behind the MFMAs of a slot, so the matrix pipe keeps running
+        // while they go out: input rows in the first four slots (their registers are free since
+        // the transforms above), the filters of an xi pair once its last MFMA has been issued.
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
+        for (int eg = 0; eg < 2; ++eg) {
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+            for (int ks = 0; ks < 4; ++ks) {
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) acc[e][nt][mt][r] = 0.0f;
-        f32x4 aA[4][NT], aB[4][NT];                 // filters of two stages in flight; component ks = k-step
-        // Unconditional loads: stages past the end re-read the last stage and are never used.
-        auto load_filters = [&](f32x4 (&a)[4][NT], int chunk) {
-            chunk = min(chunk, chEnd - 1);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int xi = 4 * wave + e;
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    a[e][nt] = *(const f32x4*)(U + (((size_t)xi * nChunksAll + chunk) * Opad + (o0 + 32 * nt + l32)) * 8 + 4 * lhi);
-            }
-        };
-        auto multiply = [&](const f32x4 (&a)[4][NT], const float* V) {
-#pragma unroll
-            for (int ks = 0; ks < KC / 2; ++ks) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float* vrow = V + ((4 * wave + e) * KC + 2 * ks + lhi) * TB + l32;
-                    float b[MT];
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) b[mt] = vrow[32 * mt];
+                for (int e = 2 * eg; e < 2 * eg + 2; ++e)
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt)
-                            acc[e][nt][mt] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[e][nt][ks], b[mt], acc[e][nt][mt], 0, 0, 0);
+                        acc[e][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[e][nt][ks], b[ks][e], acc[e][nt], 0, 0, 0);
+                if (eg == 0) {
+                    if constexpr (decltype(plainNext)::value) load_rows_plain(raw[ks], (ch + 1) * KC + 2 * ks);
+                    else load_rows_ranged(raw[ks], (ch + 1) * KC + 2 * ks);
+                } else if (ks < 2) {
+                    load_filters(f[ks], ks, next);
                 }
-            }
-        };
-        load_filters(aA, chBegin);
-        load_filters(aB, chBegin + 1);
-        wino_lds_barrier();                            // V0 holds the first stage
-        int ch = chBegin;
-        for (; ch + 1 < chEnd; ch += 2) {           // stage pairs: register sets A/B and buffers V0/V1 alternate
-            multiply(aA, V0);
-            load_filters(aA, ch + 2);
-            wino_lds_barrier();
-            multiply(aB, V1);
-            load_filters(aB, ch + 3);
-            wino_lds_barrier();
-        }
-        if (ch < chEnd) {                           // odd stage count: one more on set A
-            multiply(aA, V0);
-            wino_lds_barrier();
-        }
-        // Accumulator layout of the 32x32 MFMA: lane -> column (tile) lane%32; register r -> row
-        // (output channel) 8*(r/4) + 4*(lane/32) + r%4.  16 channels per pass go through LDS.
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                        for (int rr = 0; rr < 8; ++rr)
-                            Ms[((4 * wave + e) * 16 + 8 * (rr / 4) + 4 * lhi + (rr % 4)) * TB + 32 * mt + l32] = acc[e][nt][mt][8 * h + rr];
-                wino_lds_barrier();
-                emit_pass(nt, h);
-                wino_lds_barrier();
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-    } else {
-        // =================================== producers ===========================================
-        const int ptid = tid - PT;
-        const int tl = ptid % TB;                   // tile within the panel
-        const int cl = ptid / TB;                   // first channel-in-stage of this lane
-        int ptx, pty;
-        const bool pTileOk = tile_xy(tl, ptx, pty);
-        const int x0 = 2 * ptx - 1, y0 = 2 * pty - 1;
-        unsigned mask = 0;                          // bit 4r+s: input sample (y0+r, x0+s) exists
-        int rowOff[4], colOff[4];                   // clamped into the image: always a valid address
+        load_filters(f[2], 2, next);
+        load_filters(f[3], 3, next);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // Stages whose successor chunk is complete (all 8 channels exist) prefetch in the plain form;
+    // the last one or two of the tensor use the ranged form.
+    const int chMain = max(chBegin, min(chEnd, I / KC - 1));
+    int ch = chBegin;
+    for (; ch < chMain; ++ch) stage(ch, std::true_type{});
+    for (; ch < chEnd; ++ch) stage(ch, std::false_type{});
+
+    // ---- epilogue -----------------------------------------------------------------------------
+    // Accumulator layout of the 32x32 MFMA: lane -> column (tile) lane%32; register r -> row
+    // (output channel) 8*(r/4) + 4*(lane/32) + r%4.
+    // Each wave applies the right factor A to its row of M and parks the two results per
+    // (tile, channel) in LDS: P[row][j][channel][tile].
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float m0 = acc[0][nt][r], m1 = acc[1][nt][r], m2 = acc[2][nt][r], m3 = acc[3][nt][r];
+            const int ol = 32 * nt + 8 * (r / 4) + 4 * lhi + (r % 4);
+            P[((wave * 2 + 0) * OB + ol) * TB + l32] = m0 + m1 + m2;
+            P[((wave * 2 + 1) * OB + ol) * TB + l32] = m1 - m2 + m3;
+        }
+    }
+    // LDS-only barrier: __syncthreads() would also wait for the outstanding (unused) prefetches.
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+
+    // Left factor A^T over the four rows, bias, ReLU, store: lane -> tile tid%32, channels tid/32 + 8q.
+    const bool direct = nSplits == 1;
+    const int et = tid & 31, eo = tid >> 5;
+    const int etg = t0 + et;
+    const bool eTileOk = etg < T;
+    const int ox = eTileOk ? 2 * (etg % tilesX) : 0, oy = eTileOk ? 2 * (etg / tilesX) : 0;
+    f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
+#pragma unroll
+    for (int q = 0; q < OB / 8; ++q) {
+        const int ol = eo + 8 * q, o = o0 + ol;
+        float p[4][2];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            rowOff[r] = min(max(y0 + r, 0), H - 1) * W;
-            colOff[r] = min(max(x0 + r, 0), W - 1);
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-                if (pTileOk && y0 + r >= 0 && y0 + r < H && x0 + s >= 0 && x0 + s < W) mask |= 1u << (4 * r + s);
+            p[r][0] = P[((r * 2 + 0) * OB + ol) * TB + et];
+            p[r][1] = P[((r * 2 + 1) * OB + ol) * TB + et];
         }
-        float dA[PAIRS][16], dB[PAIRS][16];         // raw windows of two stages in flight
-        // Unconditional loads from clamped addresses; the zero padding is applied afterwards by a
-        // select.  (A load under a per-lane predicate becomes its own branch region and the compiler
-        // then waits for ALL outstanding loads at the next use, which serialises the pipeline.)
-        auto load_windows = [&](float (&d)[PAIRS][16], int chunk) {
-            chunk = min(chunk, chEnd - 1);
-#pragma unroll
-            for (int q = 0; q < PAIRS; ++q) {
-                const int c = chunk * KC + cl + q * CSTEP;
-                const float* p = in + (size_t)min(c, I - 1) * plane;
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-#pragma unroll
-                    for (int s = 0; s < 4; ++s) d[q][4 * r + s] = p[rowOff[r] + colOff[s]];
+        float y00 = p[0][0] + p[1][0] + p[2][0], y01 = p[0][1] + p[1][1] + p[2][1];
+        float y10 = p[1][0] - p[2][0] + p[3][0], y11 = p[1][1] - p[2][1] + p[3][1];
+        if (direct) {
+            if (eTileOk && o < O) {
+                if (bias) { const float bv = bias[o]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
+                if (relu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
+                wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, y00, y01, y10, y11);
             }
-        };
-        // B^T d B (left factor first, like the reference kernel), then V[xi][c][t] into LDS.
-        auto transform_store = [&](const float (&draw)[PAIRS][16], float* V, int chunk) {
-#pragma unroll
-            for (int q = 0; q < PAIRS; ++q) {
-                const unsigned mq = (chunk * KC + cl + q * CSTEP < I) ? mask : 0u;
-                float d[16], m[16];
-#pragma unroll
-                for (int k = 0; k < 16; ++k) d[k] = ((mq >> k) & 1u) ? draw[q][k] : 0.0f;   // zero padding
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    m[s]      =  d[s]     - d[8 + s];
-                    m[4 + s]  =  d[4 + s] + d[8 + s];
-                    m[8 + s]  = -d[4 + s] + d[8 + s];
-                    m[12 + s] = -d[4 + s] + d[12 + s];
-                }
-                float* dst = V + (cl + q * CSTEP) * TB + tl;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const float b0 = m[4 * r], b1 = m[4 * r + 1], b2 = m[4 * r + 2], b3 = m[4 * r + 3];
-                    dst[(4 * r + 0) * KC * TB] =  b0 - b2;
-                    dst[(4 * r + 1) * KC * TB] =  b1 + b2;
-                    dst[(4 * r + 2) * KC * TB] = -b1 + b2;
-                    dst[(4 * r + 3) * KC * TB] = -b1 + b3;
-                }
-            }
-        };
-        load_windows(dA, chBegin);
-        load_windows(dB, chBegin + 1);
-        transform_store(dA, V0, chBegin);
-        load_windows(dA, chBegin + 2);
-        wino_lds_barrier();                            // V0 holds the first stage
-        // Transforms are unconditional: past the last stage they re-transform the (clamped) last
-        // windows into the buffer nobody reads any more, which keeps the loop free of branches that
-        // would make the compiler wait for every outstanding load.
-        int ch = chBegin;
-        for (; ch + 1 < chEnd; ch += 2) {
-            transform_store(dB, V1, ch + 1);
-            load_windows(dB, ch + 3);
-            wino_lds_barrier();
-            transform_store(dA, V0, ch + 2);
-            load_windows(dA, ch + 4);
-            wino_lds_barrier();
-        }
-        if (ch < chEnd) {
-            transform_store(dB, V1, ch + 1);
-            wino_lds_barrier();
-        }
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                wino_lds_barrier();
-                emit_pass(nt, h);
-                wino_lds_barrier();
-            }
+        } else {
+            f32x4 v = {y00, y01, y10, y11};
+            wsTiles[(size_t)ol * TB + et] = v;      // whole panel, padding included: 512 B per half wave
         }
     }
 }
@@ -415,18 +353,18 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
     wino_store_tile(out + (size_t)o * H * W + (size_t)oy * W + ox, W, H, ox, oy, vec2, s[0], s[1], s[2], s[3]);
 }
 
-// variant = tile configuration (1..4, low 4 bits) | log2(number of input-channel splits) << 4
-struct WinoCfg { int mt, nt, splits; };
+// variant = output channels per workgroup (low 4 bits: 1 -> 32, 2 -> 64, 3 -> 128)
+//         | log2(number of input-channel splits) << 4
+struct WinoCfg { int nt, splits; };
 
 static bool wino_variant(int variant, WinoCfg* c) {
     const int lg = (variant >> 4) & 0xf;
     if (lg > 6 || (variant >> 8)) return false;
     c->splits = 1 << lg;
     switch (variant & 0xf) {
-        case 1: c->mt = 1; c->nt = 1; return true;
-        case 2: c->mt = 2; c->nt = 1; return true;
-        case 3: c->mt = 1; c->nt = 2; return true;
-        case 4: c->mt = 2; c->nt = 2; return true;
+        case 1: c->nt = 1; return true;
+        case 2: c->nt = 2; return true;
+        case 3: c->nt = 4; return true;
         default: return false;
     }
 }
@@ -437,7 +375,7 @@ static WinoGeom wino_geom(int W, int H, int I, int O, const WinoCfg& c) {
     WinoGeom g;
     g.tilesX = (W + 1) / 2;
     g.T = g.tilesX * ((H + 1) / 2);
-    g.nTB = ceil_div(g.T, 32 * c.mt);
+    g.nTB = ceil_div(g.T, 32);
     g.nOB = ceil_div(O, 32 * c.nt);
     g.nBlocks = g.nTB * g.nOB;
     g.nChunks = ceil_div(I, kWinoKC);
@@ -449,15 +387,15 @@ static WinoGeom wino_geom(int W, int H, int I, int O, const WinoCfg& c) {
 
 // Workspace: [splits][panel][o in panel][tile in panel] partial 2x2 tiles (float4 each).
 
-template <int MT, int NT>
+template <int NT>
 static int launch_wino(const float* in, const float* U, const float* bias, float* out, float* workspace,
                        int W, int H, int I, int O, int relu, const WinoCfg& c, hipStream_t s) {
-    constexpr int TB = 32 * MT, OB = 32 * NT;
+    constexpr int TB = 32, OB = 32 * NT;
     const WinoGeom g = wino_geom(W, H, I, O, c);
     const int gridX = ceil_div(g.nBlocks, kXcds) * kXcds;
-    const size_t ldsBytes = 2 * 16 * kWinoKC * TB * sizeof(float);
+    const size_t ldsBytes = 4 * 2 * OB * TB * sizeof(float);
     const int vec2 = ((W & 1) == 0) && (((size_t)out & 7) == 0);
-    hipLaunchKernelGGL((winograd_f23_mfma_kernel<MT, NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
+    hipLaunchKernelGGL((winograd_f23_mfma_kernel<NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
                        in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks,
                        g.chunksPerSplit, relu, vec2);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
@@ -474,20 +412,19 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
 
 using namespace drhip;
 
-// Configuration for one layer, from measurements on MI355X (256 CUs):
-//   - many tiles (>= 2048, i.e. 112x112 and larger): 32 tiles x 64 channels per workgroup -- every
-//     transformed input element then feeds twice the MFMAs;
-//   - otherwise 32 x 32 panels, and when those give fewer than ~200 workgroups (28x28, 14x14) the
-//     input channels are split until they do, keeping at least 4 stages of 8 channels per split.
+// Configuration for one layer, from measurements on MI355X (256 CUs): 64 output channels per
+// workgroup whenever the layer has them (the input transform is then shared by twice the MFMAs),
+// and the input channels split until at least ~160 workgroups exist, keeping at least 2 stages of
+// 8 channels per split.
 extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     const int T = ((W + 1) / 2) * ((H + 1) / 2);
     const int cus = num_cu();
-    if (T >= 2048 && O >= 64) return 3;
-    const int panels = ceil_div(T, 32) * ceil_div(O, 32);
+    const int code = O > 32 ? 2 : 1;
+    const int panels = ceil_div(T, 32) * ceil_div(O, code == 2 ? 64 : 32);
     const int nChunks = ceil_div(I, kWinoKC);
     int lg = 0;
-    while (lg < 4 && (panels << lg) < (3 * cus) / 4 && (nChunks >> (lg + 1)) >= 4) ++lg;
-    return 1 | (lg << 4);
+    while (lg < 5 && (panels << lg) < (5 * cus) / 8 && (nChunks >> (lg + 1)) >= 2) ++lg;
+    return code | (lg << 4);
 }
 
 extern "C" size_t drhip_conv3x3_winograd_filter_floats(int I, int O) {
@@ -500,12 +437,12 @@ extern "C" size_t drhip_conv3x3_winograd_workspace_floats(int W, int H, int I, i
     if (W <= 0 || H <= 0 || I <= 0 || O <= 0 || !wino_variant(variant, &c)) return 0;
     const WinoGeom g = wino_geom(W, H, I, O, c);
     if (g.splits <= 1) return 0;
-    return (size_t)g.splits * g.nBlocks * (32 * c.nt) * (32 * c.mt) * 4;
+    return (size_t)g.splits * g.nBlocks * (32 * c.nt) * 32 * 4;
 }
 
 extern "C" int drhip_winograd_filter_transform_f32(const float* w, float* U, int I, int O, void* stream) {
     DRHIP_REQUIRE(w && U, "drhip_winograd_filter_transform_f32: NULL tensor");
-    DRHIP_REQUIRE(I > 0 && O > 0 && (long long)(I + 7) * O * 16 < (1ll << 31), "drhip_winograd_filter_transform_f32: bad shape I=%d O=%d", I, O);
+    DRHIP_REQUIRE(I > 0 && O > 0 && (long long)(I + 7) * (O + 31) * 16 < (1ll << 29), "drhip_winograd_filter_transform_f32: bad shape I=%d O=%d", I, O);
     const int nChunks = ceil_div(I, kWinoKC);
     hipLaunchKernelGGL(winograd_filter_transform_kernel, dim3(ceil_div(nChunks * 8 * wino_opad(O), 256)), dim3(256), 0, as_stream(stream), w, U, I, O, nChunks);
     return launched("winograd_filter_transform_kernel");
@@ -516,8 +453,9 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
                                           float* workspace, void* stream) {
     DRHIP_REQUIRE(in && U && out, "drhip_conv3x3_winograd_f32: NULL tensor");
     DRHIP_REQUIRE(W > 0 && H > 0 && I > 0 && O > 0, "drhip_conv3x3_winograd_f32: bad shape %dx%dx%d -> %d", W, H, I, O);
-    DRHIP_REQUIRE((long long)W * H * I < (1ll << 31) && (long long)W * H * O < (1ll << 31) && (long long)(I + 7) * O * 16 < (1ll << 31),
-                  "drhip_conv3x3_winograd_f32: tensor too large for 32-bit indexing");
+    // byte offsets into the input and the filters are 32-bit, and 0x80000000 must lie outside both
+    DRHIP_REQUIRE((long long)W * H * I < (1ll << 29) && (long long)W * H * O < (1ll << 31) && (long long)(I + 7) * (O + 31) * 16 < (1ll << 29),
+                  "drhip_conv3x3_winograd_f32: tensor too large for 32-bit byte offsets");
     DRHIP_REQUIRE(((size_t)U & 15) == 0, "drhip_conv3x3_winograd_f32: transformed filters must be 16-byte aligned");
     if (variant == 0) {
         variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O);
@@ -529,8 +467,7 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
     DRHIP_REQUIRE(g.splits == 1 || workspace, "drhip_conv3x3_winograd_f32: variant %d splits the input channels and needs a workspace", variant);
     DRHIP_REQUIRE(g.splits <= 65535, "drhip_conv3x3_winograd_f32: too many input-channel splits");
     hipStream_t s = as_stream(stream);
-    if (c.mt == 1 && c.nt == 1) return launch_wino<1, 1>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
-    if (c.mt == 2 && c.nt == 1) return launch_wino<2, 1>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
-    if (c.mt == 1 && c.nt == 2) return launch_wino<1, 2>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
-    return launch_wino<2, 2>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
+    if (c.nt == 1) return launch_wino<1>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
+    if (c.nt == 2) return launch_wino<2>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
+    return launch_wino<4>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
 }

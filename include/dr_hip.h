@@ -100,10 +100,11 @@ size_t drhip_conv3x3_winograd_filter_floats(int I, int O);
 int drhip_winograd_filter_transform_f32(const float* w /* [I][O][3][3] */, float* U, int I, int O, void* stream);
 
 /* Fused Winograd F(2x2,3x3) convolution, stride 1, 3x3, SAME zero padding:
- * input transform B^T d B into LDS, 16 transformed-domain [tiles x I].[I x O] products on the
+ * input transform B^T d B in registers, 16 transformed-domain [tiles x I].[I x O] products on the
  * fp32 MFMA units, output transform A^T m A + bias + ReLU, edge-guarded 2x2 stores.
- * `variant` is the configuration chosen by the scheduler: low 4 bits = panel size (1..4), bits 4-7 =
- * log2 of the number of input-channel splits; 0 lets the launcher pick.  A variant that splits the
+ * `variant` is the configuration chosen by the scheduler: low 4 bits = output channels per
+ * workgroup (1: 32, 2: 64, 3: 128), bits 4-7 = log2 of the number of input-channel splits; 0 lets
+ * the launcher pick.  The input must be smaller than 2 GiB (32-bit byte offsets).  A variant that splits the
  * input channels needs `workspace` of drhip_conv3x3_winograd_workspace_floats(...) floats (scratch,
  * no initialisation needed; two launches: partial tiles, then their sum in split order); otherwise
  * workspace may be NULL.  Replaces kernel `conv2dwinograd2` and its launch
