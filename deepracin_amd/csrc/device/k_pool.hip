@@ -8,8 +8,13 @@
 // The reference does not bound-check z; a window that hangs over the last channel reads the
 // neighbouring memory there.  Here such samples read 0.0f as well.
 //
-// One lane per output element, x fastest, so a wavefront reads stride-separated but
-// line-local addresses and writes 256 contiguous bytes.
+// Small windows (2x2, 3x3): one lane per output element, x fastest, so a wavefront reads
+// stride-separated but line-local addresses and writes 256 contiguous bytes; the scan order and
+// therefore every bit of the result equal the reference's.
+// Large windows (64 samples and more, e.g. the 14x14 global average of SqueezeNet): one wavefront
+// per output element, lanes stride over the window and a butterfly reduction combines them.  The
+// maximum (and the position of its first occurrence in scan order) is still exact; an average is
+// summed in a different order than the reference's sequential loop (relative difference ~1e-7).
 #include "drhip_common.hpp"
 
 #include <cfloat>
@@ -51,6 +56,47 @@ pool_kernel(const float* __restrict__ in, float* __restrict__ out, int* __restri
     }
 }
 
+template <bool MAX, bool ARG>
+__global__ void __launch_bounds__(256)
+pool_wave_kernel(const float* __restrict__ in, float* __restrict__ out, int* __restrict__ argmax,
+                 int W, int H, int C, int Wo, int Ho, int Co,
+                 int sx, int sy, int sz, int stx, int sty, int stz) {
+    const int total = Wo * Ho * Co, n = sx * sy * sz;
+    const int lane = threadIdx.x & 63;
+    const int idx = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);     // one wavefront per output
+    if (idx >= total) return;
+    const int xo = idx % Wo, yo = (idx / Wo) % Ho, zo = idx / (Wo * Ho);
+    const int x0 = xo * stx, y0 = yo * sty, z0 = zo * stz;
+    float r = MAX ? -FLT_MAX : 0.0f;
+    int pos = 0x7fffffff, where = -1;                // scan position and flat index of the running maximum
+    for (int e = lane; e < n; e += 64) {
+        const int dx = e % sx, dy = (e / sx) % sy, dz = e / (sx * sy);
+        const int x = x0 + dx, y = y0 + dy, z = z0 + dz;
+        const bool inside = x < W && y < H && z < C;
+        const int flat = (z * H + y) * W + x;
+        const float v = inside ? in[flat] : 0.0f;
+        if (MAX) {
+            if (v > r) { r = v; pos = e; where = inside ? flat : -1; }
+        } else {
+            r += v;
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const float ro = __shfl_xor(r, m);
+        if (MAX) {
+            const int po = __shfl_xor(pos, m), wo = __shfl_xor(where, m);
+            if (ro > r || (ro == r && po < pos)) { r = ro; pos = po; where = wo; }   // first occurrence wins ties
+        } else {
+            r += ro;
+        }
+    }
+    if (lane == 0) {
+        out[idx] = MAX ? r : r / (float)n;
+        if (MAX && ARG) argmax[idx] = where;
+    }
+}
+
 }  // namespace drhip
 
 using namespace drhip;
@@ -70,6 +116,16 @@ extern "C" int drhip_pool_f32(const float* in, float* out, int* argmax_out,
     int blocks = (int)((total + block - 1) / block);
     if (blocks > 16 * num_cu()) blocks = 16 * num_cu();
     hipStream_t s = as_stream(stream);
+    if (sx * sy * sz >= 64) {                        // one wavefront per output element
+        const int wblocks = (int)((total + 3) / 4);
+        if (type == 0 && argmax_out)
+            hipLaunchKernelGGL((pool_wave_kernel<true, true>), dim3(wblocks), dim3(block), 0, s, in, out, argmax_out, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
+        else if (type == 0)
+            hipLaunchKernelGGL((pool_wave_kernel<true, false>), dim3(wblocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
+        else
+            hipLaunchKernelGGL((pool_wave_kernel<false, false>), dim3(wblocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
+        return launched("pool_wave_kernel");
+    }
     if (type == 0 && argmax_out)
         hipLaunchKernelGGL((pool_kernel<true, true>), dim3(blocks), dim3(block), 0, s, in, out, argmax_out, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
     else if (type == 0)

@@ -175,9 +175,11 @@ def test_conv1x1(lib, dev, oracle, variant, P, I, O):
     assert rel_err(dev.get(out, want2.shape), want2) <= TOL
 
 
-@pytest.mark.parametrize("W,H,C,k,s", [(56, 56, 256, 2, 2), (112, 112, 64, 3, 2), (55, 55, 7, 3, 2), (14, 14, 1000, 14, 14), (9, 7, 3, 2, 3), (5, 5, 2, 5, 1)])
+@pytest.mark.parametrize("W,H,C,k,s", [(56, 56, 256, 2, 2), (112, 112, 64, 3, 2), (55, 55, 7, 3, 2), (14, 14, 1000, 14, 14), (9, 7, 3, 2, 3), (5, 5, 2, 5, 1),
+                                         (13, 13, 5, 8, 8), (20, 17, 3, 9, 4), (30, 30, 2, 16, 16)])   # >= 64 samples: one wavefront per output
 def test_pool_bit_exact(lib, dev, oracle, W, H, C, k, s):
     x = rnd(C, H, W)                     # signed values: the zero padding is observable
+    x[:, ::3, ::2] = x[0, 0, 0]          # ties: the first maximum in scan order must win
     for kind in (0, 1):
         want, warg = oracle.pool(x, (k, k, 1), (s, s, 1), kind, want_argmax=True) if kind == 0 else (oracle.pool(x, (k, k, 1), (s, s, 1), kind), None)
         out = dev.empty(want.size)
