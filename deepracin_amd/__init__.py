@@ -142,6 +142,7 @@ def load_library(path=None):
         "drhip_event_destroy": (c_int, [vp]),
         "drhip_event_record": (c_int, [vp, vp]),
         "drhip_event_elapsed_ms": (c_int, [vp, vp, POINTER(c_float)]),
+        "drhip_stream_wait_event": (c_int, [vp, vp]),
         "drhip_conv2d_direct_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 9 + [vp]),
         "drhip_winograd_filter_transform_f32": (c_int, [vp, vp, c_int, c_int, vp]),
         "drhip_conv3x3_winograd_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 6 + [vp, vp]),

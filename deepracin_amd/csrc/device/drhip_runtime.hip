@@ -87,6 +87,11 @@ int drhip_event_elapsed_ms(void* a, void* b, float* ms) {
     return check(hipEventElapsedTime(ms, (hipEvent_t)a, (hipEvent_t)b), "hipEventElapsedTime");
 }
 
+int drhip_stream_wait_event(void* stream, void* ev) {
+    DRHIP_REQUIRE(ev, "drhip_stream_wait_event: NULL event");
+    return check(hipStreamWaitEvent(as_stream(stream), (hipEvent_t)ev, 0), "hipStreamWaitEvent");
+}
+
 int drhip_graph_capture_begin(void* stream) {
     DRHIP_REQUIRE(stream, "drhip_graph_capture_begin: the default stream cannot be captured");
     return check(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");

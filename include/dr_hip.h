@@ -58,6 +58,7 @@ int drhip_event_create(void** ev);
 int drhip_event_destroy(void* ev);
 int drhip_event_record(void* ev, void* stream);
 int drhip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms);   /* waits for ev_stop */
+int drhip_stream_wait_event(void* stream, void* ev);      /* later work on `stream` starts after `ev`; joins a capture */
 
 /* ---- launch graphs: record everything enqueued on `stream` between begin and end into an executable
  *      hipGraph and replay it with one call.  Used by dR_apply to take the per-node launch cost

@@ -197,9 +197,10 @@ def test_linearity_at_full_size(gpu):
     assert rel_err(res[2], res[0] + 2 * res[1]) <= LAYER_TOL
 
 
-def _run_many(spec, outs, inputs, graph_mode):
+def _run_many(spec, outs, inputs, graph_mode, branches=False):
     old = os.environ.get("DR_HIPGRAPH")
     os.environ["DR_HIPGRAPH"] = "1" if graph_mode else "0"
+    os.environ["DR_BRANCHES"] = "1" if branches else "0"
     try:
         with dr.Environment() as env:
             g = env.create_graph()
@@ -210,8 +211,11 @@ def _run_many(spec, outs, inputs, graph_mode):
                 configs.feed_chw(nodes[0], x)          # eager blocking copy between the replays
                 assert g.lib.dR_apply(g.ptr)
                 res.append([a.copy() for a in configs.fetch_chw(g)])   # blocking download = sync
-            used_graph = bool(ctypes.cast(g.ptr, ctypes.POINTER(_GraphTail)).contents.drGraphExec)
+            tail = ctypes.cast(g.ptr, ctypes.POINTER(_GraphTail)).contents
+            used_graph = bool(tail.drGraphExec)
+            _run_many.groups = tail.drBranchGroups
     finally:
+        os.environ.pop("DR_BRANCHES", None)
         if old is None:
             os.environ.pop("DR_HIPGRAPH", None)
         else:
@@ -227,7 +231,8 @@ class _GraphTail(ctypes.Structure):
                 ("number_of_layers", ctypes.c_int32), ("maxBufferSize", ctypes.c_int32), ("hostDebugBuffer", ctypes.c_void_p),
                 ("scheduledLayers", ctypes.c_void_p), ("allNodes", ctypes.c_void_p), ("debugLayer", ctypes.c_int),
                 ("drViewHandlers", ctypes.c_void_p), ("drLastApplyMs", ctypes.c_double), ("drGraphExec", ctypes.c_void_p),
-                ("drGraphOff", ctypes.c_int)]
+                ("drGraphOff", ctypes.c_int), ("drSideStreams", ctypes.c_void_p * 3), ("drBranchEvents", ctypes.c_void_p * 4),
+                ("drBranchGroups", ctypes.c_int)]
 
 
 @pytest.mark.parametrize("name", ["squeezenet", "vgg_conv3"])
@@ -240,6 +245,14 @@ def test_launch_graph_replays_equal_node_by_node(gpu, name):
     eager, g0 = _run_many(spec, outs, inputs, graph_mode=False)
     replay, g1 = _run_many(spec, outs, inputs, graph_mode=True)
     assert not g0 and g1, "graph mode flags: eager run used a graph=%s, graph run used a graph=%s" % (g0, g1)
+    assert _run_many.groups == 0
+    if name == "squeezenet":
+        # opt-in: the two expand convolutions of each of the 8 fire modules forked onto side streams
+        forked, g2 = _run_many(spec, outs, inputs, graph_mode=True, branches=True)
+        assert g2 and _run_many.groups == 8
+        for a, b in zip(eager, forked):
+            for x, y in zip(a, b):
+                assert np.array_equal(x, y)
     for k, (a, b) in enumerate(zip(eager, replay)):
         for x, y in zip(a, b):
             assert np.array_equal(x, y), "replay %d differs from the node-by-node pass" % k
