@@ -66,9 +66,19 @@ class ConfigStruct(Structure):
 
 
 class GraphStruct(Structure):
-    """Head of dR_Graph (include/dR_types.h)."""
+    """dR_Graph (include/dR_types.h): the reference's fields, then the ones this library appends."""
     _fields_ = [("prepared", c_int), ("swapBuffer1", c_void_p), ("swapBuffer2", c_void_p),
-                ("config", POINTER(ConfigStruct)), ("clConfig", c_void_p)]
+                ("config", POINTER(ConfigStruct)), ("clConfig", c_void_p), ("feed_layers", c_void_p),
+                ("output_layers", c_void_p), ("streamBufferHandlers", c_void_p),
+                ("number_of_layers", ctypes.c_int32), ("maxBufferSize", ctypes.c_int32), ("hostDebugBuffer", c_void_p),
+                ("scheduledLayers", c_void_p), ("allNodes", c_void_p), ("debugLayer", c_int),
+                ("drViewHandlers", c_void_p), ("drLastApplyMs", ctypes.c_double), ("drGraphExec", c_void_p),
+                ("drGraphOff", c_int), ("drSideStreams", c_void_p * 3), ("drBranchEvents", c_void_p * 4),
+                ("drBranchGroups", c_int)]
+
+
+def graph_struct(graph):
+    return ctypes.cast(graph.ptr, POINTER(GraphStruct)).contents
 
 
 def node_struct(node):
@@ -143,6 +153,9 @@ def load_library(path=None):
         "drhip_event_record": (c_int, [vp, vp]),
         "drhip_event_elapsed_ms": (c_int, [vp, vp, POINTER(c_float)]),
         "drhip_stream_wait_event": (c_int, [vp, vp]),
+        "drhip_timing_begin": (c_int, []),
+        "drhip_timing_count": (c_int, []),
+        "drhip_timing_end": (c_int, [POINTER(c_float), c_int, POINTER(c_int)]),
         "drhip_conv2d_direct_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 9 + [vp]),
         "drhip_winograd_filter_transform_f32": (c_int, [vp, vp, c_int, c_int, vp]),
         "drhip_conv3x3_winograd_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 6 + [vp, vp]),

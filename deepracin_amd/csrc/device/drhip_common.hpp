@@ -2,9 +2,11 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdio>
+#include <vector>
 
 #include "dr_hip.h"
 
@@ -32,6 +34,34 @@ inline int launched(const char* kernel) { return check(hipGetLastError(), kernel
 inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
 
 constexpr int kWave = 64;   // CDNA wavefront width
+
+// Per-thread record of kernel execution times (drhip_timing_begin / drhip_timing_end).  While it is
+// on, every launch carries its own start and stop event (hipExtLaunchKernelGGL attaches them to the
+// dispatch packet), so the span is the kernel alone -- no extra packets between the kernels, which
+// is what events recorded between launches would put there.
+struct LaunchTimer {
+    bool on = false;
+    size_t used = 0;                   // events handed out since drhip_timing_begin
+    std::vector<hipEvent_t> events;    // [2*i] start, [2*i+1] stop of launch i
+};
+LaunchTimer& launch_timer();
+
+// Every kernel of this library is launched through here.
+template <typename Kernel, typename... Args>
+inline void launch(Kernel kernel, dim3 grid, dim3 block, size_t ldsBytes, hipStream_t stream, Args... args) {
+    LaunchTimer& t = launch_timer();
+    if (!t.on) {
+        hipLaunchKernelGGL(kernel, grid, block, ldsBytes, stream, args...);
+        return;
+    }
+    while (t.events.size() < t.used + 2) {
+        hipEvent_t e;
+        if (hipEventCreate(&e) != hipSuccess) { hipLaunchKernelGGL(kernel, grid, block, ldsBytes, stream, args...); return; }
+        t.events.push_back(e);
+    }
+    hipExtLaunchKernelGGL(kernel, grid, block, ldsBytes, stream, t.events[t.used], t.events[t.used + 1], 0, args...);
+    t.used += 2;
+}
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 

@@ -13,6 +13,11 @@ char* error_slot() {
 static int g_num_cu = 256;
 int num_cu() { return g_num_cu; }
 
+LaunchTimer& launch_timer() {
+    static thread_local LaunchTimer t;
+    return t;
+}
+
 __global__ void fill_f32_kernel(float* __restrict__ dst, float value, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -87,6 +92,28 @@ int drhip_event_elapsed_ms(void* a, void* b, float* ms) {
     return check(hipEventElapsedTime(ms, (hipEvent_t)a, (hipEvent_t)b), "hipEventElapsedTime");
 }
 
+int drhip_timing_begin(void) {
+    LaunchTimer& t = launch_timer();
+    t.used = 0;
+    t.on = true;
+    return DRHIP_OK;
+}
+
+int drhip_timing_count(void) { return (int)(launch_timer().used / 2); }
+
+int drhip_timing_end(float* ms, int capacity, int* count) {
+    LaunchTimer& t = launch_timer();
+    t.on = false;
+    const int n = (int)(t.used / 2);
+    if (count) *count = n;
+    DRHIP_REQUIRE(n == 0 || (ms && capacity >= n), "drhip_timing_end: room for %d launches needed, %d given", n, capacity);
+    for (int i = 0; i < n; ++i) {
+        if (int rc = check(hipEventSynchronize(t.events[2 * i + 1]), "hipEventSynchronize")) return rc;
+        if (int rc = check(hipEventElapsedTime(&ms[i], t.events[2 * i], t.events[2 * i + 1]), "hipEventElapsedTime")) return rc;
+    }
+    return DRHIP_OK;
+}
+
 int drhip_stream_wait_event(void* stream, void* ev) {
     DRHIP_REQUIRE(ev, "drhip_stream_wait_event: NULL event");
     return check(hipStreamWaitEvent(as_stream(stream), (hipEvent_t)ev, 0), "hipStreamWaitEvent");
@@ -152,7 +179,7 @@ int drhip_fill_f32(float* dst, float value, size_t n, void* stream) {
     const int block = 256;
     size_t blocks = (n + block - 1) / block;
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(fill_f32_kernel, dim3((unsigned)blocks), dim3(block), 0, as_stream(stream), dst, value, n);
+    launch(fill_f32_kernel, dim3((unsigned)blocks), dim3(block), 0, as_stream(stream), dst, value, n);
     return launched("fill_f32_kernel");
 }
 

@@ -136,7 +136,7 @@ extern "C" int drhip_conv1x1_f32(const float* in, const float* w, const float* b
     DRHIP_REQUIRE(variant == 1 || variant == 2 || variant == 4 || variant == 8, "drhip_conv1x1_f32: unknown variant %d (waves per tile: 1, 2, 4, 8)", variant);
     const int nPT = ceil_div(P, 32), nOT = ceil_div(O, 32);
     const size_t ldsBytes = variant > 1 ? (size_t)variant * 32 * kC1Pad * sizeof(float) : 0;
-    hipLaunchKernelGGL(conv1x1_mfma_kernel, dim3(nPT * nOT), dim3(64 * variant), ldsBytes, as_stream(stream),
+    launch(conv1x1_mfma_kernel, dim3(nPT * nOT), dim3(64 * variant), ldsBytes, as_stream(stream),
                        in, w, bias, out, P, I, O, nPT, relu);
     return launched("conv1x1_mfma_kernel");
 }

@@ -111,9 +111,9 @@ static int launch_direct(const float* in, const float* w, const float* bias, flo
     const size_t ldsBytes = (size_t)CC * perChannel * sizeof(float);
     dim3 grid(tilesX * tilesY, ceil_div(O, OCT)), block(kDirThreads);
     if (kw == 3 && kh == 3)
-        hipLaunchKernelGGL((conv_direct_kernel<OCT, 3, 3>), grid, block, ldsBytes, s, in, w, bias, out, W, H, I, O, Wo, Ho, kw, kh, sx, sy, CC, tilesX, relu);
+        launch((conv_direct_kernel<OCT, 3, 3>), grid, block, ldsBytes, s, in, w, bias, out, W, H, I, O, Wo, Ho, kw, kh, sx, sy, CC, tilesX, relu);
     else
-        hipLaunchKernelGGL((conv_direct_kernel<OCT, 0, 0>), grid, block, ldsBytes, s, in, w, bias, out, W, H, I, O, Wo, Ho, kw, kh, sx, sy, CC, tilesX, relu);
+        launch((conv_direct_kernel<OCT, 0, 0>), grid, block, ldsBytes, s, in, w, bias, out, W, H, I, O, Wo, Ho, kw, kh, sx, sy, CC, tilesX, relu);
     return launched("conv_direct_kernel");
 }
 

@@ -188,14 +188,14 @@ extern "C" int drhip_fc_f32(const float* x, const float* Wt, const float* bias, 
     dim3 grid(p.panels, p.slices), block(kFcThreads);
     hipStream_t s = as_stream(stream);
     if (p.vec == 4)
-        hipLaunchKernelGGL((fc_gemv_kernel<4>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
+        launch((fc_gemv_kernel<4>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
     else if (p.vec == 2)
-        hipLaunchKernelGGL((fc_gemv_kernel<2>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
+        launch((fc_gemv_kernel<2>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
     else
-        hipLaunchKernelGGL((fc_gemv_kernel<1>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
+        launch((fc_gemv_kernel<1>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
     if (int rc = launched("fc_gemv_kernel")) return rc;
     if (p.slices > 1) {
-        hipLaunchKernelGGL(fc_reduce_kernel, dim3(ceil_div(N, 256)), dim3(256), 0, s, partials, bias, y, N, p.slices, relu);
+        launch(fc_reduce_kernel, dim3(ceil_div(N, 256)), dim3(256), 0, s, partials, bias, y, N, p.slices, relu);
         return launched("fc_reduce_kernel");
     }
     return DRHIP_OK;
@@ -205,6 +205,6 @@ extern "C" int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, in
     DRHIP_REQUIRE(src && dst && src != dst, "drhip_fc_permute_rows_f32: NULL or aliased matrices");
     DRHIP_REQUIRE(W > 0 && H > 0 && C > 0 && N > 0, "drhip_fc_permute_rows_f32: bad shape");
     DRHIP_REQUIRE((long long)W * H * C < (1ll << 31), "drhip_fc_permute_rows_f32: K too large");
-    hipLaunchKernelGGL(fc_permute_rows_kernel, dim3(W * H * C), dim3(256), 0, as_stream(stream), src, dst, W, H, C, N);
+    launch(fc_permute_rows_kernel, dim3(W * H * C), dim3(256), 0, as_stream(stream), src, dst, W, H, C, N);
     return launched("fc_permute_rows_kernel");
 }

@@ -56,7 +56,7 @@ extern "C" int drhip_copy3d_f32(const float* src, int sW, int sH, int sx0, int s
     const int total = w * h * c, block = 256;
     int blocks = ceil_div(total, block);
     if (blocks > 16 * num_cu()) blocks = 16 * num_cu();
-    hipLaunchKernelGGL(copy3d_kernel, dim3(blocks), dim3(block), 0, as_stream(stream),
+    launch(copy3d_kernel, dim3(blocks), dim3(block), 0, as_stream(stream),
                        src, sW, sH, sx0, sy0, sz0, dst, dW, dH, dx0, dy0, dz0, w, h, c);
     return launched("copy3d_kernel");
 }
@@ -68,6 +68,6 @@ extern "C" int drhip_scalar_op_f32(const float* x, float* y, size_t n, int op, f
     const int block = 256;
     size_t blocks = (n + block - 1) / block;
     if (blocks > (size_t)16 * num_cu()) blocks = (size_t)16 * num_cu();
-    hipLaunchKernelGGL(scalar_op_kernel, dim3((unsigned)blocks), dim3(block), 0, as_stream(stream), x, y, n, op, s);
+    launch(scalar_op_kernel, dim3((unsigned)blocks), dim3(block), 0, as_stream(stream), x, y, n, op, s);
     return launched("scalar_op_kernel");
 }

@@ -119,18 +119,18 @@ extern "C" int drhip_pool_f32(const float* in, float* out, int* argmax_out,
     if (sx * sy * sz >= 64) {                        // one wavefront per output element
         const int wblocks = (int)((total + 3) / 4);
         if (type == 0 && argmax_out)
-            hipLaunchKernelGGL((pool_wave_kernel<true, true>), dim3(wblocks), dim3(block), 0, s, in, out, argmax_out, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
+            launch((pool_wave_kernel<true, true>), dim3(wblocks), dim3(block), 0, s, in, out, argmax_out, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
         else if (type == 0)
-            hipLaunchKernelGGL((pool_wave_kernel<true, false>), dim3(wblocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
+            launch((pool_wave_kernel<true, false>), dim3(wblocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
         else
-            hipLaunchKernelGGL((pool_wave_kernel<false, false>), dim3(wblocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
+            launch((pool_wave_kernel<false, false>), dim3(wblocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
         return launched("pool_wave_kernel");
     }
     if (type == 0 && argmax_out)
-        hipLaunchKernelGGL((pool_kernel<true, true>), dim3(blocks), dim3(block), 0, s, in, out, argmax_out, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
+        launch((pool_kernel<true, true>), dim3(blocks), dim3(block), 0, s, in, out, argmax_out, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
     else if (type == 0)
-        hipLaunchKernelGGL((pool_kernel<true, false>), dim3(blocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
+        launch((pool_kernel<true, false>), dim3(blocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
     else
-        hipLaunchKernelGGL((pool_kernel<false, false>), dim3(blocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
+        launch((pool_kernel<false, false>), dim3(blocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
     return launched("pool_kernel");
 }

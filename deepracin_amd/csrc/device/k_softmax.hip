@@ -65,6 +65,6 @@ using namespace drhip;
 extern "C" int drhip_softmax_f32(const float* x, float* y, int n, void* stream) {
     DRHIP_REQUIRE(x && y, "drhip_softmax_f32: NULL tensor");
     DRHIP_REQUIRE(n > 0, "drhip_softmax_f32: n = %d", n);
-    hipLaunchKernelGGL(softmax_kernel, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, y, n);
+    launch(softmax_kernel, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, y, n);
     return launched("softmax_kernel");
 }

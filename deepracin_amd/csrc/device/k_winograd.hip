@@ -395,13 +395,13 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
     const int gridX = ceil_div(g.nBlocks, kXcds) * kXcds;
     const size_t ldsBytes = 4 * 2 * OB * TB * sizeof(float);
     const int vec2 = ((W & 1) == 0) && (((size_t)out & 7) == 0);
-    hipLaunchKernelGGL((winograd_f23_mfma_kernel<NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
+    launch((winograd_f23_mfma_kernel<NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
                        in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks,
                        g.chunksPerSplit, relu, vec2);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
     if (g.splits > 1) {
         const int total = g.nBlocks * OB * TB;
-        hipLaunchKernelGGL(winograd_split_reduce_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s,
+        launch(winograd_split_reduce_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s,
                            workspace, bias, out, W, H, O, g.tilesX, g.T, g.nTB, g.nBlocks, TB, OB, g.splits, relu, vec2);
         return launched("winograd_split_reduce_kernel");
     }
@@ -444,7 +444,7 @@ extern "C" int drhip_winograd_filter_transform_f32(const float* w, float* U, int
     DRHIP_REQUIRE(w && U, "drhip_winograd_filter_transform_f32: NULL tensor");
     DRHIP_REQUIRE(I > 0 && O > 0 && (long long)(I + 7) * (O + 31) * 16 < (1ll << 29), "drhip_winograd_filter_transform_f32: bad shape I=%d O=%d", I, O);
     const int nChunks = ceil_div(I, kWinoKC);
-    hipLaunchKernelGGL(winograd_filter_transform_kernel, dim3(ceil_div(nChunks * 8 * wino_opad(O), 256)), dim3(256), 0, as_stream(stream), w, U, I, O, nChunks);
+    launch(winograd_filter_transform_kernel, dim3(ceil_div(nChunks * 8 * wino_opad(O), 256)), dim3(256), 0, as_stream(stream), w, U, I, O, nChunks);
     return launched("winograd_filter_transform_kernel");
 }
 

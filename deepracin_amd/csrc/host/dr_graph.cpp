@@ -5,6 +5,7 @@
 #include "dr_internal.hpp"
 
 #include <chrono>
+#include <vector>
 
 using namespace dr;
 
@@ -262,37 +263,37 @@ gboolean dR_apply(dR_Graph* net) {
         }
     }
 
+    // profilingGPU: every kernel launch carries its own start/stop events (drhip_timing_*), and a
+    // node's time is the sum of its kernels -- the per-kernel profiling the reference took from
+    // OpenCL events (src/dR_clwrap.c:718-741).
     const int nNodes = net->scheduledLayers->length;
-    if (profGPU && cc->hipNumEvents < nNodes + 1) {
-        void** ev = (void**)realloc(cc->hipEvents, sizeof(void*) * (size_t)(nNodes + 1));
-        if (!ev) return FALSE;
-        cc->hipEvents = ev;
-        for (; cc->hipNumEvents < nNodes + 1; cc->hipNumEvents++)
-            if (device_failed(net, drhip_event_create(&cc->hipEvents[cc->hipNumEvents]), "dR_apply(profile)")) return FALSE;
-    }
-    if (profGPU) drhip_event_record(cc->hipEvents[0], cc->hipStream);
+    std::vector<int> firstLaunch;
+    if (profGPU) { firstLaunch.reserve((size_t)nNodes + 1); drhip_timing_begin(); }
 
-    int pos = 0;
-    for (dR_ListElement* e = net->scheduledLayers->first; e; e = e->next, ++pos) {
+    for (dR_ListElement* e = net->scheduledLayers->first; e; e = e->next) {
         dR_Node* node = (dR_Node*)e->element;
+        if (profGPU) firstLaunch.push_back(drhip_timing_count());
         if (!node->compute(net, node)) {
             say("Execution of layer %d failed \n", node->layerID);
+            if (profGPU) drhip_timing_end(NULL, 0, NULL);
             return FALSE;
         }
-        if (profGPU) drhip_event_record(cc->hipEvents[pos + 1], cc->hipStream);
         if (node->layerID == net->debugLayer && net->hostDebugBuffer)
             dR_downloadArray(net, (gchar*)"", node->outputBuf->bufptr, 0,
                              (size_t)node->oshape.s0 * node->oshape.s1 * sizeof(float), net->hostDebugBuffer);
     }
     if (profGPU) {
-        pos = 0;
+        firstLaunch.push_back(drhip_timing_count());
+        std::vector<float> ms((size_t)firstLaunch.back() + 1);
+        int launches = 0;
+        if (device_failed(net, drhip_timing_end(ms.data(), (int)ms.size(), &launches), "dR_apply(profile)")) return FALSE;
+        int pos = 0;
         cc->totalKernelGPUTime = 0;
         for (dR_ListElement* e = net->scheduledLayers->first; e; e = e->next, ++pos) {
-            float ms = 0.f;
-            if (device_failed(net, drhip_event_elapsed_ms(cc->hipEvents[pos], cc->hipEvents[pos + 1], &ms), "dR_apply(profile)"))
-                return FALSE;
-            ((dR_Node*)e->element)->drLastKernelMs = ms;
-            cc->totalKernelGPUTime += ms;
+            float sum = 0.f;
+            for (int k = firstLaunch[pos]; k < firstLaunch[pos + 1]; ++k) sum += ms[k];
+            ((dR_Node*)e->element)->drLastKernelMs = sum;
+            cc->totalKernelGPUTime += sum;
         }
         say("GPU Profiling: Sum of all kernel run times: %2.3fms \n", cc->totalKernelGPUTime);   // unconditional, like the reference
         cc->sumTotalKernelGPUTime += cc->totalKernelGPUTime;
@@ -326,10 +327,6 @@ void dR_cleanup(dR_Graph* net, gboolean cleanupcl) {
 gboolean dR_cleanupCL(dR_Graph* net) {
     dR_ClConfig* cc = net->clConfig;
     if (!cc->clContext || cc->cleanupDone) return TRUE;
-    for (int i = 0; i < cc->hipNumEvents; ++i) drhip_event_destroy(cc->hipEvents[i]);
-    free(cc->hipEvents);
-    cc->hipEvents = NULL;
-    cc->hipNumEvents = 0;
     if (cc->hipOwnsStream && cc->hipStream) drhip_stream_destroy(cc->hipStream);
     cc->hipStream = NULL;
     free(cc->clDeviceName);

@@ -145,8 +145,6 @@ struct dR_ClConfig {
 
     /* ---- additions of this build ---- */
     void*               hipStream;          /* hipStream_t all work of this graph is ordered on */
-    void**              hipEvents;          /* hipEvent_t[hipNumEvents]: node boundaries of a profiled dR_apply */
-    gint                hipNumEvents;
     gint                hipNumCU;           /* compute units of the device (256 on MI355X) */
     gint                hipLdsBytes;        /* LDS bytes per workgroup limit */
     gboolean            hipOwnsStream;

@@ -58,6 +58,14 @@ int drhip_event_create(void** ev);
 int drhip_event_destroy(void* ev);
 int drhip_event_record(void* ev, void* stream);
 int drhip_event_elapsed_ms(void* ev_start, void* ev_stop, float* ms);   /* waits for ev_stop */
+/* Kernel execution times of the calling thread's launches: between drhip_timing_begin and
+ * drhip_timing_end every kernel launch of this library carries its own start/stop event pair, so
+ * ms[i] is the device time of launch i alone (what OpenCL's per-kernel profiling events gave the
+ * reference, src/dR_clwrap.c:718-741).  drhip_timing_count = launches recorded so far;
+ * drhip_timing_end waits for them and switches the recording off.  Not for use under capture. */
+int drhip_timing_begin(void);
+int drhip_timing_count(void);
+int drhip_timing_end(float* ms, int capacity, int* count);
 int drhip_stream_wait_event(void* stream, void* ev);      /* later work on `stream` starts after `ev`; joins a capture */
 
 /* ---- launch graphs: record everything enqueued on `stream` between begin and end into an executable

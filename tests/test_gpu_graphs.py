@@ -211,7 +211,7 @@ def _run_many(spec, outs, inputs, graph_mode, branches=False):
                 configs.feed_chw(nodes[0], x)          # eager blocking copy between the replays
                 assert g.lib.dR_apply(g.ptr)
                 res.append([a.copy() for a in configs.fetch_chw(g)])   # blocking download = sync
-            tail = ctypes.cast(g.ptr, ctypes.POINTER(_GraphTail)).contents
+            tail = dr.graph_struct(g)
             used_graph = bool(tail.drGraphExec)
             _run_many.groups = tail.drBranchGroups
     finally:
@@ -221,18 +221,6 @@ def _run_many(spec, outs, inputs, graph_mode, branches=False):
         else:
             os.environ["DR_HIPGRAPH"] = old
     return res, used_graph
-
-
-class _GraphTail(ctypes.Structure):
-    """dR_Graph (include/dR_types.h) up to the launch-graph fields."""
-    _fields_ = [("prepared", ctypes.c_int), ("swapBuffer1", ctypes.c_void_p), ("swapBuffer2", ctypes.c_void_p),
-                ("config", ctypes.c_void_p), ("clConfig", ctypes.c_void_p), ("feed_layers", ctypes.c_void_p),
-                ("output_layers", ctypes.c_void_p), ("streamBufferHandlers", ctypes.c_void_p),
-                ("number_of_layers", ctypes.c_int32), ("maxBufferSize", ctypes.c_int32), ("hostDebugBuffer", ctypes.c_void_p),
-                ("scheduledLayers", ctypes.c_void_p), ("allNodes", ctypes.c_void_p), ("debugLayer", ctypes.c_int),
-                ("drViewHandlers", ctypes.c_void_p), ("drLastApplyMs", ctypes.c_double), ("drGraphExec", ctypes.c_void_p),
-                ("drGraphOff", ctypes.c_int), ("drSideStreams", ctypes.c_void_p * 3), ("drBranchEvents", ctypes.c_void_p * 4),
-                ("drBranchGroups", ctypes.c_int)]
 
 
 @pytest.mark.parametrize("name", ["squeezenet", "vgg_conv3"])
