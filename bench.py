@@ -41,7 +41,10 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch of the dominant kernel from `rocprofv3 --pmc FETCH_SIZE` / `--pmc WRITE_SIZE`
 # runs of this script, scaled by what the same counters read for a copy of known size; the
 # commands and the per-layer figures are in profiles/.  Keyed by (workload, kernel group).
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
+    ("vgg16", "winograd"): 26340.6 * 1024,      # profiles/vgg16_hbm_traffic.md: fetch 239 513 + write 102 915 KiB over 13 launches
+    ("vgg16", "fc"): 162372.1 * 1024,
+}
 
 
 class _QuietStdout:
