@@ -133,9 +133,6 @@ __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, 
 constexpr unsigned kBufferFlags = 0x00020000u;      // dword 3 of a gfx9 raw buffer resource (32-bit data format)
 constexpr unsigned kOutOfRange = 0x80000000u;       // byte offset no resource of at most 2 GiB contains
 
-__device__ inline float buf_load(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)voffset, (int)soffset, 0));
-}
 __device__ inline f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset) {
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voffset, (int)soffset, 0));
 }
@@ -174,31 +171,37 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     const int x0 = 2 * tx - 1, y0 = 2 * ty - 1;
     const int rowA = wave, rowB = (wave < 2) ? 2 : 1;
     const float sgn = (wave == 1) ? 1.0f : -1.0f;
-    unsigned offA[4], offB[4];
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-        const int x = x0 + s, ya = y0 + rowA, yb = y0 + rowB;
-        const bool xOk = tileOk && x >= 0 && x < W;
-        offA[s] = (xOk && ya >= 0 && ya < H) ? 4u * (unsigned)(lhi * plane + ya * W + x) : kOutOfRange;
-        offB[s] = (xOk && yb >= 0 && yb < H) ? 4u * (unsigned)(lhi * plane + yb * W + x) : kOutOfRange;
-    }
+    // One 16-byte load per row from the (4-byte aligned) address of its first sample.  Rows outside
+    // the image carry the out-of-range offset as a whole; samples beyond the left or right edge come
+    // back as the neighbouring row's pixels and are zeroed by three selects after the rows have been
+    // combined (the second sample, x = 2*tx, always exists).  A negative offset would zero the whole
+    // load, and only image tile 0 has one (x = -1 in row 0): that one lane loads from x = 0 instead
+    // and shifts its combined samples up by one (three more selects for everybody; a branch around
+    // them costs more in register copies than it saves).
+    const bool shifted = tg == 0;
+    const int xLoad = shifted ? 0 : x0;
+    const int yaRow = y0 + rowA, ybRow = y0 + rowB;
+    const unsigned offVA = (tileOk && yaRow >= 0 && yaRow < H) ? 4u * (unsigned)(lhi * plane + yaRow * W + xLoad) : kOutOfRange;
+    const unsigned offVB = (tileOk && ybRow >= 0 && ybRow < H) ? 4u * (unsigned)(lhi * plane + ybRow * W + xLoad) : kOutOfRange;
+    const bool c0ok = x0 >= 0, c2ok = x0 + 2 < W, c3ok = x0 + 3 < W;
+
     // Window rows of channels cbase + lhi.  "Ranged" form: the resource starts at channel cbase and
     // ends with the tensor, so channels >= I read 0 without touching memory (ragged last chunk,
     // prefetch past the end).  "Plain" form for chunks known to lie inside the tensor: one resource
     // for the whole tensor, the channel offset travels in the scalar offset (a resource that changes
     // inside the loop makes the compiler wait for all outstanding loads at the loop head).
     const __amdgpu_buffer_rsrc_t rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kBufferFlags);
-    auto load_rows_plain = [&](float (&d)[8], int cbase) {
-        const unsigned soff = 4u * (unsigned)(cbase * plane);
+    auto load_rows = [&](float (&d)[8], __amdgpu_buffer_rsrc_t r, unsigned soff) {
+        const f32x4 a = buf_load4(r, offVA, soff), b = buf_load4(r, offVB, soff);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) { d[s] = buf_load(rIn, offA[s], soff); d[4 + s] = buf_load(rIn, offB[s], soff); }
+        for (int s = 0; s < 4; ++s) { d[s] = a[s]; d[4 + s] = b[s]; }
     };
+    auto load_rows_plain = [&](float (&d)[8], int cbase) { load_rows(d, rIn, 4u * (unsigned)(cbase * plane)); };
     auto load_rows_ranged = [&](float (&d)[8], int cbase) {
         const int left = max(I - cbase, 0);
         const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(in + (size_t)min(cbase, I) * plane), 0,
                                                                              left * plane * 4, kBufferFlags);
-#pragma unroll
-        for (int s = 0; s < 4; ++s) { d[s] = buf_load(r, offA[s], 0); d[4 + s] = buf_load(r, offB[s], 0); }
+        load_rows(d, r, 0u);
     };
     // filters of one xi for a whole stage: component ks of the 16-byte load = k-step ks
     const __amdgpu_buffer_rsrc_t rU = __builtin_amdgcn_make_buffer_rsrc((void*)U, 0, 16 * nChunksAll * Opad * 8 * 4, kBufferFlags);
@@ -234,6 +237,11 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
             float m[4];
 #pragma unroll
             for (int s = 0; s < 4; ++s) m[s] = fmaf(sgn, raw[ks][4 + s], raw[ks][s]);   // exact: sgn is +-1
+            const float s1 = shifted ? m[0] : m[1], s2 = shifted ? m[1] : m[2], s3 = shifted ? m[2] : m[3];
+            m[0] = c0ok ? m[0] : 0.0f;
+            m[1] = s1;
+            m[2] = c2ok ? s2 : 0.0f;
+            m[3] = c3ok ? s3 : 0.0f;
             b[ks][0] = m[0] - m[2];
             b[ks][1] = m[1] + m[2];
             b[ks][2] = m[2] - m[1];
@@ -326,15 +334,21 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
 
 // out[o][2x2 tile] = act(bias[o] + sum over splits of the partial tile), splits added in order.
 // One lane per (o, tile); partials are [split][panel][o in panel][tile in panel] float4.
+// Workgroup b works for panel (b % 8) * perXcd + ..., i.e. on the XCD whose workgroups wrote that
+// panel's partial tiles a moment ago: they are still in that XCD's L2.
 __global__ void __launch_bounds__(256)
 winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restrict__ bias, float* __restrict__ out,
-                             int W, int H, int O, int tilesX, int T, int nTB, int nBlocks, int TB, int OB,
+                             int W, int H, int O, int tilesX, int T, int nTB, int nBlocks, int perXcd, int TB, int OB,
                              int nSplits, int relu, int vec2) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;      // over nBlocks * OB * TB
-    if (idx >= nBlocks * OB * TB) return;
-    const int tLocal = idx % TB, ol = (idx / TB) % OB, panel = idx / (TB * OB);
+    const int blocksPerPanel = (TB * OB) / 256;
+    const int j = blockIdx.x / kXcds;
+    const int panel = (blockIdx.x % kXcds) * perXcd + j / blocksPerPanel;
+    if (j / blocksPerPanel >= perXcd || panel >= nBlocks) return;
+    const int within = (j % blocksPerPanel) * 256 + threadIdx.x;    // (o in panel) * TB + tile in panel
+    const int tLocal = within % TB, ol = within / TB;
     const int o = (panel / nTB) * OB + ol, tg = (panel % nTB) * TB + tLocal;
     if (o >= O || tg >= T) return;
+    const size_t idx = (size_t)panel * TB * OB + within;
     const f32x4* p = (const f32x4*)ws + idx;
     const size_t splitStride = (size_t)nBlocks * OB * TB;
     f32x4 s = {0.f, 0.f, 0.f, 0.f};
@@ -400,9 +414,9 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
                        g.chunksPerSplit, relu, vec2);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
     if (g.splits > 1) {
-        const int total = g.nBlocks * OB * TB;
-        launch(winograd_split_reduce_kernel, dim3(ceil_div(total, 256)), dim3(256), 0, s,
-                           workspace, bias, out, W, H, O, g.tilesX, g.T, g.nTB, g.nBlocks, TB, OB, g.splits, relu, vec2);
+        const int perXcd = gridX / kXcds;
+        launch(winograd_split_reduce_kernel, dim3(gridX * (OB * TB / 256)), dim3(256), 0, s,
+               workspace, bias, out, W, H, O, g.tilesX, g.T, g.nTB, g.nBlocks, perXcd, TB, OB, g.splits, relu, vec2);
         return launched("winograd_split_reduce_kernel");
     }
     return DRHIP_OK;
