@@ -427,21 +427,18 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
 using namespace drhip;
 
 // Configuration for one layer, from measurements on MI355X (256 CUs):
-//   - 64 output channels per workgroup (the input transform is shared by twice the MFMAs) unless
-//     the layer is tiny (SqueezeNet's expand convolutions: at most 64 input channels on 56x56 or
-//     smaller), where 32-channel panels give more workgroups and finish sooner;
-//   - the input channels are split until at least ~160 workgroups exist, keeping 2 stages of 8
-//     channels per split (tiny layers: 1 stage, at most 4 splits, none below 32 input channels).
+//   - 32 output channels per workgroup; 64 only for layers with very many tiles (224x224), where
+//     the panels alone give several workgroups per CU and sharing the input transform pays;
+//   - the input channels are split until at least ~160 workgroups exist, keeping at least 2 stages
+//     of 8 channels per split.
 extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     const int T = ((W + 1) / 2) * ((H + 1) / 2);
     const int cus = num_cu();
-    const bool tiny = T < 1024 && I <= 64;
-    const int code = (O > 32 && !tiny) ? 2 : 1;
+    const int code = (O > 32 && T >= 8192) ? 2 : 1;
     const int panels = ceil_div(T, 32) * ceil_div(O, code == 2 ? 64 : 32);
     const int nChunks = ceil_div(I, kWinoKC);
-    const int minStages = tiny ? 1 : 2, maxLg = tiny ? (nChunks >= 4 ? 2 : 0) : 5;
     int lg = 0;
-    while (lg < maxLg && (panels << lg) < (5 * cus) / 8 && (nChunks >> (lg + 1)) >= minStages) ++lg;
+    while (lg < 5 && (panels << lg) < (5 * cus) / 8 && (nChunks >> (lg + 1)) >= 2) ++lg;
     return code | (lg << 4);
 }
 
