@@ -131,6 +131,7 @@ __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, 
 // KS > 1: every split stores its partial (pre-bias) 2x2 tiles, tile-major, to the workspace and
 // winograd_split_reduce_kernel sums them in split order, adds the bias and applies ReLU.
 constexpr unsigned kBufferFlags = 0x00020000u;      // dword 3 of a gfx9 raw buffer resource (32-bit data format)
+constexpr int kEpiRelu = DRHIP_EPILOGUE_RELU, kEpiMaxPool2 = DRHIP_EPILOGUE_MAXPOOL2;   // bits of the `relu` argument
 constexpr unsigned kOutOfRange = 0x80000000u;       // byte offset no resource of at most 2 GiB contains
 
 __device__ inline f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset) {
@@ -322,8 +323,11 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
         if (direct) {
             if (eTileOk && o < O) {
                 if (bias) { const float bv = bias[o]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
-                if (relu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
-                wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, y00, y01, y10, y11);
+                if (relu & kEpiRelu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
+                if (relu & kEpiMaxPool2)        // W, H even: the tile is one window of a 2x2/2 max pool
+                    out[(size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1)] = fmaxf(fmaxf(y00, y01), fmaxf(y10, y11));
+                else
+                    wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, y00, y01, y10, y11);
             }
         } else {
             f32x4 v = {y00, y01, y10, y11};
@@ -362,9 +366,12 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
     }
     for (; sp < nSplits; ++sp) s += p[(size_t)sp * splitStride];
     if (bias) s += bias[o];
-    if (relu) { s[0] = fmaxf(s[0], 0.f); s[1] = fmaxf(s[1], 0.f); s[2] = fmaxf(s[2], 0.f); s[3] = fmaxf(s[3], 0.f); }
+    if (relu & kEpiRelu) { s[0] = fmaxf(s[0], 0.f); s[1] = fmaxf(s[1], 0.f); s[2] = fmaxf(s[2], 0.f); s[3] = fmaxf(s[3], 0.f); }
     const int ox = 2 * (tg % tilesX), oy = 2 * (tg / tilesX);
-    wino_store_tile(out + (size_t)o * H * W + (size_t)oy * W + ox, W, H, ox, oy, vec2, s[0], s[1], s[2], s[3]);
+    if (relu & kEpiMaxPool2)
+        out[(size_t)o * ((H >> 1) * (W >> 1)) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1)] = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+    else
+        wino_store_tile(out + (size_t)o * H * W + (size_t)oy * W + ox, W, H, ox, oy, vec2, s[0], s[1], s[2], s[3]);
 }
 
 // variant = output channels per workgroup (low 4 bits: 1 -> 32, 2 -> 64, 3 -> 128)
@@ -472,6 +479,8 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
     DRHIP_REQUIRE((long long)W * H * I < (1ll << 29) && (long long)W * H * O < (1ll << 31) && (long long)(I + 7) * (O + 31) * 16 < (1ll << 29),
                   "drhip_conv3x3_winograd_f32: tensor too large for 32-bit byte offsets");
     DRHIP_REQUIRE(((size_t)U & 15) == 0, "drhip_conv3x3_winograd_f32: transformed filters must be 16-byte aligned");
+    DRHIP_REQUIRE((relu & ~(DRHIP_EPILOGUE_RELU | DRHIP_EPILOGUE_MAXPOOL2)) == 0, "drhip_conv3x3_winograd_f32: unknown epilogue flags %d", relu);
+    DRHIP_REQUIRE(!(relu & DRHIP_EPILOGUE_MAXPOOL2) || ((W | H) & 1) == 0, "drhip_conv3x3_winograd_f32: the fused 2x2 max pool needs even W and H (got %dx%d)", W, H);
     if (variant == 0) {
         variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O);
         if (!workspace) variant &= 0xf;            // no workspace offered: stay unsplit

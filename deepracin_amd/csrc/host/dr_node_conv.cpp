@@ -128,7 +128,7 @@ gboolean conv_compute(dR_Graph* net, dR_Node* node) {
     dR_Conv2d_Data* c = conv_of(node);
     dR_Node* src = first_input(node);
     const float* in = dev_out(src);
-    float* out = dev_out(node);
+    float* out = dev_out(node);         // with drFusedPool this is the pooling node's buffer
     const float* w = (const float*)c->weightsBuf;
     const float* b = c->useBias ? (const float*)c->biasBuf : NULL;
     const int W = c->ishape.s0, H = c->ishape.s1, I = c->shape.s2, O = c->shape.s3;
@@ -136,7 +136,9 @@ gboolean conv_compute(dR_Graph* net, dR_Node* node) {
     int rc;
     switch (c->algo) {
         case drConvWinograd:
-            rc = drhip_conv3x3_winograd_f32(in, w, b, out, W, H, I, O, relu, c->variant, (float*)c->workspaceBuf, stream_of(net));
+            rc = drhip_conv3x3_winograd_f32(in, w, b, out, W, H, I, O,
+                                            (relu ? DRHIP_EPILOGUE_RELU : 0) | (c->drFusedPool ? DRHIP_EPILOGUE_MAXPOOL2 : 0),
+                                            c->variant, (float*)c->workspaceBuf, stream_of(net));
             break;
         case drConv1x1Gemm:
             rc = drhip_conv1x1_f32(in, w, b, out, W * H, I, O, relu, c->variant, stream_of(net));

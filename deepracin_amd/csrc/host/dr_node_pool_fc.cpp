@@ -48,6 +48,7 @@ gboolean pool_schedule(dR_Graph* net, dR_Node* node) {
 
 gboolean pool_compute(dR_Graph* net, dR_Node* node) {
     dR_Pooling_Data* p = pool_of(node);
+    if (p->drFused) return TRUE;        // the convolution in front stored the pooled tensor already
     int rc = drhip_pool_f32(dev_out(first_input(node)), dev_out(node), NULL, p->ishape.s0, p->ishape.s1, p->ishape.s2,
                             p->shape.s1, p->shape.s2, p->shape.s3, p->stride.s1, p->stride.s2, p->stride.s3,
                             (int)p->poolingType, stream_of(net));

@@ -50,6 +50,25 @@ bool concat_can_fuse(const dR_Node* c) {
     return !ins.empty();
 }
 
+// A 2x2 / stride-2 max pool directly behind a Winograd convolution: every 2x2 output tile of the
+// convolution is one pooling window, so the convolution's epilogue can store the maximum and the
+// full-resolution tensor never exists.  Only when nobody else wants that tensor.
+dR_Node* pool_fusable_producer(const dR_Node* p) {
+    if (p->type != tPooling) return nullptr;
+    const char* env = getenv("DR_FUSE_POOL");
+    if (env && strcmp(env, "0") == 0) return nullptr;
+    const dR_Pooling_Data* pd = (const dR_Pooling_Data*)p->layer;
+    if (pd->poolingType != tMax || pd->shape.s1 != 2 || pd->shape.s2 != 2 || pd->shape.s3 != 1 ||
+        pd->stride.s1 != 2 || pd->stride.s2 != 2 || pd->stride.s3 != 1) return nullptr;
+    std::vector<dR_Node*> ins = nodes_of(p->previous_layers);
+    if (ins.size() != 1) return nullptr;
+    dR_Node* c = ins[0];
+    if (c->type != tConv2d || ((const dR_Conv2d_Data*)c->layer)->algo != drConvWinograd) return nullptr;
+    if (c->output || c->outputBuf || !c->next_layers || c->next_layers->length != 1) return nullptr;
+    if ((c->oshape.s0 | c->oshape.s1) & 1) return nullptr;
+    return c;
+}
+
 }  // namespace
 
 extern "C" {
@@ -164,6 +183,12 @@ gboolean dR_planBuffers(dR_Graph* net) {
     // 1. which concat nodes absorb their producers
     std::map<dR_Node*, std::pair<dR_Node*, int>> parent;   // producer -> (concat, float offset)
     for (dR_Node* n : sched) {
+        if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drFusedPool = FALSE;
+        if (n->type == tPooling) {
+            dR_Node* c = pool_fusable_producer(n);
+            ((dR_Pooling_Data*)n->layer)->drFused = c != nullptr;
+            if (c) { ((dR_Conv2d_Data*)c->layer)->drFusedPool = TRUE; parent[c] = std::make_pair(n, 0); }
+        }
         if (n->type != tConcat) continue;
         dR_Concat_Data* cd = (dR_Concat_Data*)n->layer;
         cd->drFused = concat_can_fuse(n);

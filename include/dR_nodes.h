@@ -43,6 +43,8 @@ struct dR_Conv2d_Data {
     gint                variant;        /* tile configuration id understood by the drhip_* launcher */
     gint                winogradn;      /* always 2: F(2x2,3x3) */
     cl_mem              workspaceBuf;   /* split-K scratch of the Winograd kernel, NULL when the layer is not split */
+    gboolean            drFusedPool;    /* set by the buffer planner: the node's only consumer is a 2x2/2 max pool and
+                                           this node writes the pooled tensor straight into that node's buffer */
 };
 
 /*
@@ -71,6 +73,7 @@ struct dR_Pooling_Data {
     dR_PoolingType  poolingType;
     gchar**         shaderSrc;  /* unused placeholder */
     gboolean        useLMEM;    /* unused placeholder */
+    gboolean        drFused;    /* set by the buffer planner: the producing convolution already pooled; compute() is a no-op */
 };
 
 /* Output dims = ceil(in/stride); window anchored top-left at (x*stx, y*sty, z*stz), no leading

@@ -116,8 +116,14 @@ int drhip_winograd_filter_transform_f32(const float* w /* [I][O][3][3] */, float
  * the launcher pick.  The input must be smaller than 2 GiB (32-bit byte offsets).  A variant that splits the
  * input channels needs `workspace` of drhip_conv3x3_winograd_workspace_floats(...) floats (scratch,
  * no initialisation needed; two launches: partial tiles, then their sum in split order); otherwise
- * workspace may be NULL.  Replaces kernel `conv2dwinograd2` and its launch
+ * workspace may be NULL.  `relu` is a set of epilogue flags: DRHIP_EPILOGUE_RELU (1) and
+ * DRHIP_EPILOGUE_MAXPOOL2 (2): `out` is then [O][H/2][W/2] and receives the 2x2 / stride-2 maximum
+ * of every output tile instead of the tile (what a following max-pooling node with window and stride
+ * (2,2,1) would compute, src/dR_nodes_pooling.c:277-401; W and H must be even).
+ * Replaces kernel `conv2dwinograd2` and its launch
  * (Kernels/dR_winograd2.cl:23-254, src/dR_nodes_conv2d.c:1009-1132). */
+#define DRHIP_EPILOGUE_RELU     1
+#define DRHIP_EPILOGUE_MAXPOOL2 2
 int drhip_conv3x3_winograd_f32(const float* in, const float* U, const float* bias, float* out,
                                int W, int H, int I, int O, int relu, int variant,
                                float* workspace, void* stream);

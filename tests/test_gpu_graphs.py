@@ -113,6 +113,25 @@ def test_config3_vgg_conv3_block(oracle, gpu):
     del want
 
 
+def test_maxpool_fused_into_convolution(oracle, gpu):
+    """With only the final tensor requested, the last convolution of the block stores the pooled
+    tensor itself (no pooling launch); the numbers equal the unfused run bit for bit."""
+    spec, feeds, fused = run_config("vgg_conv3")
+    _, _, plain = run_config("vgg_conv3", env_vars={"DR_FUSE_POOL": "0"})
+    assert np.array_equal(fused[4], plain[4]) and fused[4].shape == (256, 28, 28)
+    want = oracle.run_spec(spec, feeds)
+    assert rel_err(fused[4], want[4]) <= LAYER_TOL
+    # the pooling node of the fused run launches nothing
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes = configs.build_graph(g, spec, [4])
+        dr.prepare(g)
+        configs.feed_chw(nodes[0], feeds[0])
+        dr.graph_config(g).profilingGPU = 1
+        assert g.lib.dR_apply(g.ptr)
+        assert dr.node_struct(nodes[4]).drLastKernelMs == 0.0 and dr.node_struct(nodes[3]).drLastKernelMs > 0.0
+
+
 def test_config4_squeezenet(oracle, gpu):
     spec, feeds, got = run_config("squeezenet", outputs=all_compute_nodes)
     want = check_layers(oracle, spec, feeds, got)

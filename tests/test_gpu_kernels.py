@@ -136,6 +136,29 @@ def test_winograd_conv(lib, dev, oracle, variant, W, H, I, O):
     assert rel_err(dev.get(out, want2.shape), want2) <= TOL
 
 
+@pytest.mark.parametrize("variant", [1, 2, 0x11, 0x22])
+@pytest.mark.parametrize("W,H,I,O", [(56, 56, 64, 64), (28, 12, 24, 40), (2, 2, 1, 1), (224, 224, 3, 64)])
+def test_winograd_fused_maxpool(lib, dev, oracle, variant, W, H, I, O):
+    """Epilogue flag 2: the kernel stores the 2x2/2 maximum of every output tile -- bit for bit what
+    the pooling kernel makes of the kernel's own unpooled output."""
+    x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
+    U, _ = wino_filters(lib, dev, w)
+    ws = wino_workspace(lib, dev, W, H, I, O, variant)
+    xd, bd = dev.put(x), dev.put(b)
+    for relu in (1, 0):
+        full = dev.empty(O * H * W)
+        ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, full, W, H, I, O, relu, variant, ws, None))
+        want = oracle.pool(dev.get(full, (O, H, W)), (2, 2, 1), (2, 2, 1), 0)
+        pooled = dev.empty(want.size)
+        ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, pooled, W, H, I, O, relu | 2, variant, ws, None))
+        assert np.array_equal(dev.get(pooled, want.shape), want)
+        ref = oracle.pool(oracle.conv_winograd(x, w, b, relu=bool(relu)), (2, 2, 1), (2, 2, 1), 0)
+        assert rel_err(dev.get(pooled, want.shape), ref) <= TOL
+    p = dev.empty(64)
+    assert lib.drhip_conv3x3_winograd_f32(p, U, None, p, 3, 4, I, O, 2, 1, None, None) == -1      # odd width
+    assert lib.drhip_conv3x3_winograd_f32(p, U, None, p, 4, 4, I, O, 4, 1, None, None) == -1      # unknown flag
+
+
 def test_winograd_auto_variant_vgg_shapes(lib, dev, oracle):
     for (W, I, O) in [(56, 128, 256), (28, 256, 512), (14, 512, 512)]:
         x, w, b = np.abs(rnd(I, W, W)), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
