@@ -153,6 +153,9 @@ def load_library(path=None):
         "drhip_event_record": (c_int, [vp, vp]),
         "drhip_event_elapsed_ms": (c_int, [vp, vp, POINTER(c_float)]),
         "drhip_stream_wait_event": (c_int, [vp, vp]),
+        "drhip_fc_slices": (c_int, [c_int, c_int]),
+        "drhip_fc_ex_f32": (c_int, [vp, vp, vp, vp, vp, vp, c_int, c_int, c_int, c_int, vp]),
+        "drhip_softmax_ex_f32": (c_int, [vp, vp, vp, c_int, vp]),
         "drhip_timing_begin": (c_int, []),
         "drhip_timing_count": (c_int, []),
         "drhip_timing_end": (c_int, [POINTER(c_float), c_int, POINTER(c_int)]),

@@ -8,6 +8,10 @@
 //   - a workgroup (4 waves) owns a panel of CBW = 64*VEC columns and a slice of rows; its waves take
 //     64-row chunks round-robin and keep 8-16 row loads (8-16 KiB per wave) in flight;
 //   - x for a 64-row chunk is loaded once, one element per lane, and broadcast with v_readlane;
+//   - the input vector may arrive unfinished, as the partial sums a previous GEMV left behind
+//     (drhip_deferred_vec): a wave then sums the slices of its 64 rows itself, in slice order, adds
+//     the bias and applies ReLU - bit for bit what the reduce kernel would have stored, without
+//     the launch (a ~4 us kernel between two GEMVs of 13 and 7 us);
 //   - split-K: the grid is (column panels) x (row slices), sized to a few workgroups per CU; each
 //     workgroup writes one partial row and a second, tiny kernel sums the partials in slice order,
 //     adds the bias and applies ReLU (the same two-step shape as the reference; no device-scope
@@ -59,11 +63,29 @@ static FcPlan fc_plan(int K, int N) {
 
 // Partial GEMV of one (column panel, row slice).  slices == 1: writes y directly (bias, ReLU).
 // Otherwise writes partials[slice][n]; fc_reduce_kernel finishes.
-template <int VEC>
+// Element `row` of an activation vector left as partial sums: slices added in order, then bias, ReLU.
+__device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {
+    const float* pp = d.partials + row;
+    float s = 0.0f;
+    int sl = 0;
+    for (; sl + 8 <= d.slices; sl += 8) {           // 8 independent loads in flight, summed in slice order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = pp[(size_t)(sl + u) * d.n];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; sl < d.slices; ++sl) s += pp[(size_t)sl * d.n];
+    if (d.bias) s += d.bias[row];
+    if (d.relu) s = fmaxf(s, 0.0f);
+    return s;
+}
+
+template <int VEC, bool DEFERRED>
 __global__ void __launch_bounds__(kFcThreads)
-fc_gemv_kernel(const float* __restrict__ x, const float* __restrict__ Wt, const float* __restrict__ bias,
-               float* __restrict__ y, float* __restrict__ partials,
-               int K, int N, int rowsPerSlice, int relu) {
+fc_gemv_kernel(const float* __restrict__ x, drhip_deferred_vec xdef, const float* __restrict__ Wt,
+               const float* __restrict__ bias, float* __restrict__ y, float* __restrict__ partials,
+               int K, int N, int rowsPerSlice, int relu, int defer) {
     typedef typename VecT<VEC>::type vec_t;
     constexpr int CBW = kWave * VEC;
     __shared__ float red[kFcWaves][CBW];
@@ -82,7 +104,7 @@ fc_gemv_kernel(const float* __restrict__ x, const float* __restrict__ Wt, const 
 
     for (int r0 = rowBegin + wave * kWave; r0 < rowEnd; r0 += kFcWaves * kWave) {
         const int rows = min(kWave, rowEnd - r0);
-        const float xraw = x[min(r0 + lane, K - 1)];
+        const float xraw = DEFERRED ? deferred_element(xdef, min(r0 + lane, K - 1)) : x[min(r0 + lane, K - 1)];
         const float xl = (lane < rows) ? xraw : 0.0f;
         const float* wp = Wt + (size_t)r0 * N + col;
         if (rows == kWave) {
@@ -177,28 +199,48 @@ extern "C" size_t drhip_fc_scratch_floats(int K, int N) {
     return p.slices > 1 ? (size_t)p.slices * (size_t)N : 0;
 }
 
-extern "C" int drhip_fc_f32(const float* x, const float* Wt, const float* bias, float* y,
-                            float* partials, int K, int N, int relu, void* stream) {
-    DRHIP_REQUIRE(x && Wt && y, "drhip_fc_f32: NULL pointer");
+extern "C" int drhip_fc_slices(int K, int N) {
+    if (K <= 0 || N <= 0) return 0;
+    return fc_plan(K, N).slices;
+}
+
+template <int VEC>
+static void launch_gemv(bool deferred, dim3 grid, hipStream_t s, const float* x, const drhip_deferred_vec& xd, const float* Wt,
+                        const float* bias, float* y, float* partials, int K, int N, int rowsPerSlice, int relu, int defer) {
+    if (deferred) launch((fc_gemv_kernel<VEC, true>), grid, dim3(kFcThreads), 0, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
+    else launch((fc_gemv_kernel<VEC, false>), grid, dim3(kFcThreads), 0, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
+}
+
+extern "C" int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, const float* Wt, const float* bias, float* y,
+                               float* partials, int K, int N, int relu, int defer, void* stream) {
+    DRHIP_REQUIRE((x || xdef) && Wt && (y || defer), "drhip_fc_f32: NULL pointer");
     DRHIP_REQUIRE(K > 0 && N > 0, "drhip_fc_f32: bad shape K=%d N=%d", K, N);
+    DRHIP_REQUIRE(!xdef || (xdef->partials && xdef->slices > 0 && xdef->n == K),
+                  "drhip_fc_f32: deferred input must carry partial sums of a vector of length K=%d", K);
     FcPlan p = fc_plan(K, N);
     DRHIP_REQUIRE(p.slices == 1 || partials, "drhip_fc_f32: this shape is split over %d row slices and needs the partials scratch", p.slices);
+    DRHIP_REQUIRE(!defer || p.slices > 1, "drhip_fc_f32: only a layer that is split over row slices can leave its sum unfinished");
     DRHIP_REQUIRE(((size_t)Wt % (4 * p.vec)) == 0, "drhip_fc_f32: weight matrix not aligned for %d-wide loads", p.vec);
     DRHIP_REQUIRE(p.slices <= 65535, "drhip_fc_f32: too many row slices");
-    dim3 grid(p.panels, p.slices), block(kFcThreads);
+    dim3 grid(p.panels, p.slices);
     hipStream_t s = as_stream(stream);
-    if (p.vec == 4)
-        launch((fc_gemv_kernel<4>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
-    else if (p.vec == 2)
-        launch((fc_gemv_kernel<2>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
-    else
-        launch((fc_gemv_kernel<1>), grid, block, 0, s, x, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu);
+    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0};
+    const drhip_deferred_vec& xd = xdef ? *xdef : none;
+    if (p.vec == 4) launch_gemv<4>(xdef != nullptr, grid, s, x, xd, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu, defer);
+    else if (p.vec == 2) launch_gemv<2>(xdef != nullptr, grid, s, x, xd, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu, defer);
+    else launch_gemv<1>(xdef != nullptr, grid, s, x, xd, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu, defer);
     if (int rc = launched("fc_gemv_kernel")) return rc;
-    if (p.slices > 1) {
+    if (p.slices > 1 && !defer) {
         launch(fc_reduce_kernel, dim3(ceil_div(N, 256)), dim3(256), 0, s, partials, bias, y, N, p.slices, relu);
         return launched("fc_reduce_kernel");
     }
     return DRHIP_OK;
+}
+
+extern "C" int drhip_fc_f32(const float* x, const float* Wt, const float* bias, float* y,
+                            float* partials, int K, int N, int relu, void* stream) {
+    DRHIP_REQUIRE(x && y, "drhip_fc_f32: NULL pointer");
+    return drhip_fc_ex_f32(x, nullptr, Wt, bias, y, partials, K, N, relu, 0, stream);
 }
 
 extern "C" int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, int H, int C, int N, void* stream) {

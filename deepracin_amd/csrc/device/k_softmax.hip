@@ -22,12 +22,25 @@ __device__ inline float wave_sum(float v) {
     return v;
 }
 
+// xdef.partials != NULL: the logits arrive as the partial sums of the GEMV in front (slices added
+// in order, then its bias and ReLU); they are finished into y first, which then serves as x.
 __global__ void __launch_bounds__(kSoftmaxThreads)
-softmax_kernel(const float* __restrict__ x, float* __restrict__ y, int n) {
+softmax_kernel(const float* x, drhip_deferred_vec xdef, float* y, int n) {     // no __restrict__: x may become y
     __shared__ float red[kSoftmaxThreads / kWave];
     __shared__ float bcast;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     constexpr int nwaves = kSoftmaxThreads / kWave;
+    if (xdef.partials) {
+        for (int i = tid; i < n; i += kSoftmaxThreads) {
+            const float* pp = xdef.partials + i;
+            float s = 0.0f;
+            for (int sl = 0; sl < xdef.slices; ++sl) s += pp[(size_t)sl * xdef.n];
+            if (xdef.bias) s += xdef.bias[i];
+            if (xdef.relu) s = fmaxf(s, 0.0f);
+            y[i] = s;                           // every lane re-reads only the elements it wrote itself
+        }
+        x = y;
+    }
 
     float m = -FLT_MAX;
     for (int i = tid; i < n; i += kSoftmaxThreads) m = fmaxf(m, x[i]);
@@ -62,9 +75,16 @@ softmax_kernel(const float* __restrict__ x, float* __restrict__ y, int n) {
 
 using namespace drhip;
 
-extern "C" int drhip_softmax_f32(const float* x, float* y, int n, void* stream) {
-    DRHIP_REQUIRE(x && y, "drhip_softmax_f32: NULL tensor");
+extern "C" int drhip_softmax_ex_f32(const float* x, const drhip_deferred_vec* xdef, float* y, int n, void* stream) {
+    DRHIP_REQUIRE((x || xdef) && y, "drhip_softmax_f32: NULL tensor");
     DRHIP_REQUIRE(n > 0, "drhip_softmax_f32: n = %d", n);
-    launch(softmax_kernel, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, y, n);
+    DRHIP_REQUIRE(!xdef || (xdef->partials && xdef->slices > 0 && xdef->n == n), "drhip_softmax_f32: deferred input must carry partial sums of a vector of length %d", n);
+    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0};
+    launch(softmax_kernel, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, xdef ? *xdef : none, y, n);
     return launched("softmax_kernel");
+}
+
+extern "C" int drhip_softmax_f32(const float* x, float* y, int n, void* stream) {
+    DRHIP_REQUIRE(x, "drhip_softmax_f32: NULL tensor");
+    return drhip_softmax_ex_f32(x, nullptr, y, n, stream);
 }

@@ -145,11 +145,25 @@ gboolean fc_fill(dR_Graph* net, dR_Node* node) {
     return ok;
 }
 
+// Where an FC node that skipped its finishing kernel left its output.
+drhip_deferred_vec deferred_output_of(dR_Node* producer) {
+    dR_FC_Data* p = fc_of(producer);
+    drhip_deferred_vec d;
+    d.partials = (const float*)p->partialsBuf;
+    d.bias = p->useBias ? (const float*)p->biasBuf : NULL;
+    d.slices = drhip_fc_slices(p->shape.s0, p->shape.s1);
+    d.n = p->shape.s1;
+    d.relu = p->activation == tReLU;
+    return d;
+}
+
 gboolean fc_compute(dR_Graph* net, dR_Node* node) {
     dR_FC_Data* f = fc_of(node);
-    int rc = drhip_fc_f32(dev_out(first_input(node)), (const float*)f->weightsBuf, f->useBias ? (const float*)f->biasBuf : NULL,
-                          dev_out(node), (float*)f->partialsBuf, f->shape.s0, f->shape.s1,
-                          f->activation == tReLU, stream_of(net));
+    drhip_deferred_vec xdef;
+    if (f->drDeferredInput) xdef = deferred_output_of(f->drDeferredInput);
+    int rc = drhip_fc_ex_f32(dev_out(first_input(node)), f->drDeferredInput ? &xdef : NULL, (const float*)f->weightsBuf,
+                             f->useBias ? (const float*)f->biasBuf : NULL, dev_out(node), (float*)f->partialsBuf,
+                             f->shape.s0, f->shape.s1, f->activation == tReLU, f->drDeferReduce, stream_of(net));
     return !device_failed(net, rc, "deepRACIN:FullyConnected");
 }
 
@@ -211,7 +225,10 @@ gboolean softmax_propagate(dR_Graph* net, dR_Node* node) {
 
 gboolean softmax_compute(dR_Graph* net, dR_Node* node) {
     dR_Softmax_Data* s = (dR_Softmax_Data*)node->layer;
-    int rc = drhip_softmax_f32(dev_out(first_input(node)), dev_out(node), s->ishape.s0 * s->ishape.s1 * s->ishape.s2, stream_of(net));
+    drhip_deferred_vec xdef;
+    if (s->drDeferredInput) xdef = deferred_output_of(s->drDeferredInput);
+    int rc = drhip_softmax_ex_f32(dev_out(first_input(node)), s->drDeferredInput ? &xdef : NULL, dev_out(node),
+                                  s->ishape.s0 * s->ishape.s1 * s->ishape.s2, stream_of(net));
     return !device_failed(net, rc, "deepRACIN:softmax");
 }
 

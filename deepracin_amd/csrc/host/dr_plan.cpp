@@ -182,6 +182,24 @@ gboolean dR_planBuffers(dR_Graph* net) {
 
     // 1. which concat nodes absorb their producers
     std::map<dR_Node*, std::pair<dR_Node*, int>> parent;   // producer -> (concat, float offset)
+    // FC -> FC and FC -> softmax: the consumer sums the producer's split-K partials while it loads
+    // its input, the producer's finishing kernel is not launched (DR_FUSE_FC=0 keeps it).
+    for (dR_Node* n : sched) {
+        if (n->type == tFullyConnected) { ((dR_FC_Data*)n->layer)->drDeferReduce = FALSE; ((dR_FC_Data*)n->layer)->drDeferredInput = nullptr; }
+        if (n->type == tSoftmax) ((dR_Softmax_Data*)n->layer)->drDeferredInput = nullptr;
+    }
+    const char* fuseFc = getenv("DR_FUSE_FC");
+    for (dR_Node* n : sched) {
+        if (n->type != tFullyConnected || (fuseFc && strcmp(fuseFc, "0") == 0)) continue;
+        dR_FC_Data* fd = (dR_FC_Data*)n->layer;
+        if (n->output || n->outputBuf || !n->next_layers || n->next_layers->length != 1) continue;
+        if (drhip_fc_slices(fd->shape.s0, fd->shape.s1) <= 1) continue;
+        dR_Node* c = nodes_of(n->next_layers)[0];
+        if (c->type == tFullyConnected) ((dR_FC_Data*)c->layer)->drDeferredInput = n;
+        else if (c->type == tSoftmax) ((dR_Softmax_Data*)c->layer)->drDeferredInput = n;
+        else continue;
+        fd->drDeferReduce = TRUE;
+    }
     for (dR_Node* n : sched) {
         if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drFusedPool = FALSE;
         if (n->type == tPooling) {

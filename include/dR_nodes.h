@@ -96,6 +96,8 @@ struct dR_FC_Data {
     dR_ActivationType   activation;
     /* gfx950 plan */
     cl_mem              partialsBuf;    /* split-K partial sums, NULL when the layer is not split */
+    gboolean            drDeferReduce;  /* set by the buffer planner: the only consumer (FC or softmax) sums the partials itself */
+    dR_Node*            drDeferredInput; /* set by the buffer planner: the FC node in front left its output as partial sums */
 };
 
 /* y[n] = act(b[n] + sum_k x_hwc[k] * W[k][n]); shape = (K, N); K must equal W*H*C of the input. */
@@ -110,6 +112,7 @@ struct dR_Softmax_Data {
     dR_Shape3   ishape;
     cl_kernel   clKernelComputeExp;     /* unused placeholder */
     gfloat*     expsHost;               /* unused placeholder: the sum stays on the device */
+    dR_Node*    drDeferredInput;        /* set by the buffer planner: the FC node in front left its output as partial sums */
 };
 
 /* p = exp(x) / sum(exp(x)) over all W*H*C elements of the input. */

@@ -164,6 +164,21 @@ int drhip_pool_f32(const float* in, float* out, int* argmax_out,
 size_t drhip_fc_scratch_floats(int K, int N);
 int drhip_fc_f32(const float* x, const float* Wt, const float* bias, float* y,
                  float* partials, int K, int N, int relu, void* stream);
+/* Chains of GEMVs without the small kernels in between.  With `defer` != 0 a layer that is split
+ * over row slices (drhip_fc_slices(K,N) > 1) stops after the partial sums: y is not written, and
+ * the consumer is told where the sums are through a drhip_deferred_vec: element k of that vector is
+ * act(bias[k] + sum_{s < slices} partials[s*n + k]), slices added in order - the value, bit for bit,
+ * that the finishing kernel would have stored.  drhip_fc_ex_f32 and drhip_softmax_ex_f32 accept
+ * such a vector as their input (`xdef` != NULL; x is then ignored).  No counterpart in the
+ * reference, which always runs its second kernel (src/dR_nodes_fc.c:239-275). */
+typedef struct drhip_deferred_vec {
+    const float* partials;   /* [slices][n] */
+    const float* bias;       /* [n] or NULL */
+    int slices, n, relu;
+} drhip_deferred_vec;
+int drhip_fc_slices(int K, int N);
+int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, const float* Wt, const float* bias, float* y,
+                    float* partials, int K, int N, int relu, int defer, void* stream);
 /* dst[k_chw][n] = src[k_hwc][n] with k_hwc = (y*W + x)*C + z for k_chw = (z*H + y)*W + x. */
 int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, int H, int C, int N, void* stream);
 
@@ -171,6 +186,7 @@ int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, int H, int C,
  * shuffles.  Replaces computeExp + host-side sum + mulScalar (src/dR_nodes_math.c:620-678,
  * Kernels/dR_math.cl:216-227,295-305). */
 int drhip_softmax_f32(const float* x, float* y, int n, void* stream);
+int drhip_softmax_ex_f32(const float* x, const drhip_deferred_vec* xdef, float* y, int n, void* stream);
 
 /* ---- data movement nodes ------------------------------------------------------------------------
  * copy3d: dst[(z+dz0)][y+dy0][x+dx0] = src[(z+sz0)][y+sy0][x+sx0] for a (w,h,c) box; serves Concat

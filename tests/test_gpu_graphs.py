@@ -132,6 +132,38 @@ def test_maxpool_fused_into_convolution(oracle, gpu):
         assert dr.node_struct(nodes[4]).drLastKernelMs == 0.0 and dr.node_struct(nodes[3]).drLastKernelMs > 0.0
 
 
+def test_fc_chain_fused(oracle, gpu):
+    """FC -> FC -> softmax: the finishing kernels of the two GEMVs disappear into their consumers
+    (3 launches instead of 5) and the probabilities do not change by a bit."""
+    rng = np.random.default_rng(5)
+    spec = [{"op": "feed", "shape": (4, 4, 64)},
+            {"op": "fc", "in": 0, "w": (rng.standard_normal((1024, 2048)) * 0.04).astype(np.float32), "b": (rng.standard_normal(2048) * 0.01).astype(np.float32), "relu": True},
+            {"op": "fc", "in": 1, "w": (rng.standard_normal((2048, 1000)) * 0.03).astype(np.float32), "b": (rng.standard_normal(1000) * 0.01).astype(np.float32), "relu": False},
+            {"op": "softmax", "in": 2}]
+    x = rng.random((64, 4, 4), dtype=np.float32)
+    res, launches = {}, {}
+    for mode in ("1", "0"):
+        os.environ["DR_FUSE_FC"] = mode
+        try:
+            with dr.Environment() as env:
+                g = env.create_graph()
+                nodes = configs.build_graph(g, spec, [3])
+                dr.prepare(g)
+                configs.feed_chw(nodes[0], x)
+                assert g.lib.dR_apply(g.ptr) and g.lib.dR_apply(g.ptr)          # captured pass, then its replay
+                res[mode] = configs.fetch_chw(g)[0].copy()
+                dr.graph_config(g).profilingGPU = 1
+                assert g.lib.dR_apply(g.ptr)
+                launches[mode] = g.lib.drhip_timing_count()
+                assert np.array_equal(configs.fetch_chw(g)[0], res[mode])
+        finally:
+            os.environ.pop("DR_FUSE_FC", None)
+    assert launches == {"1": 3, "0": 5}
+    assert np.array_equal(res["1"], res["0"])
+    want = oracle.run_spec(spec, {0: x})
+    assert rel_err(res["1"], want[3]) <= LAYER_TOL and int(res["1"].argmax()) == int(want[3].argmax())
+
+
 def test_config4_squeezenet(oracle, gpu):
     spec, feeds, got = run_config("squeezenet", outputs=all_compute_nodes)
     want = check_layers(oracle, spec, feeds, got)

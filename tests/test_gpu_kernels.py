@@ -245,6 +245,45 @@ def test_fc(lib, dev, oracle, C, H, W, N, relu):
         first = got
 
 
+class DeferredVec(ctypes.Structure):
+    """drhip_deferred_vec (include/dr_hip.h)."""
+    _fields_ = [("partials", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("slices", ctypes.c_int), ("n", ctypes.c_int), ("relu", ctypes.c_int)]
+
+
+def test_fc_chain_without_finishing_kernels(lib, dev, oracle):
+    """FC -> FC -> softmax where each consumer sums the producer's split-K partials itself: every
+    result equals the one of the three separate calls bit for bit."""
+    K, N1, N2 = 1024, 2048, 1000
+    x, W1, b1 = np.abs(rnd(K)), rnd(K, N1, scale=np.sqrt(2.0 / K)), rnd(N1, scale=0.01)
+    W2, b2 = rnd(N1, N2, scale=np.sqrt(2.0 / N1)), rnd(N2, scale=0.01)
+    xd, W1d, b1d, W2d, b2d = dev.put(x), dev.put(W1), dev.put(b1), dev.put(W2), dev.put(b2)
+    s1, s2 = lib.drhip_fc_slices(K, N1), lib.drhip_fc_slices(N1, N2)
+    assert s1 > 1 and s2 > 1 and lib.drhip_fc_scratch_floats(K, N1) == s1 * N1
+    p1, p2 = dev.empty(s1 * N1), dev.empty(s2 * N2)
+    y1, y2, prob = dev.empty(N1), dev.empty(N2), dev.empty(N2)
+    # plain chain
+    ok(lib, lib.drhip_fc_f32(xd, W1d, b1d, y1, p1, K, N1, 1, None))
+    ok(lib, lib.drhip_fc_f32(y1, W2d, b2d, y2, p2, N1, N2, 0, None))
+    ok(lib, lib.drhip_softmax_f32(y2, prob, N2, None))
+    want2, wantp = dev.get(y2, (N2,)), dev.get(prob, (N2,))
+    assert rel_err(want2, oracle.fc(oracle.fc(x.reshape(K, 1, 1), W1, b1, relu=True), W2, b2, relu=False).reshape(-1)) <= TOL
+    # deferred chain: y1 and y2 are never written
+    q1, q2, prob2 = dev.empty(s1 * N1), dev.empty(s2 * N2), dev.empty(N2)
+    ok(lib, lib.drhip_fc_ex_f32(xd, None, W1d, b1d, None, q1, K, N1, 1, 1, None))
+    d1 = DeferredVec(q1.value, b1d.value, s1, N1, 1)
+    y2b = dev.empty(N2)
+    ok(lib, lib.drhip_fc_ex_f32(None, ctypes.byref(d1), W2d, b2d, y2b, q2, N1, N2, 0, 0, None))
+    assert np.array_equal(dev.get(y2b, (N2,)), want2)
+    ok(lib, lib.drhip_fc_ex_f32(None, ctypes.byref(d1), W2d, b2d, None, q2, N1, N2, 0, 1, None))
+    d2 = DeferredVec(q2.value, b2d.value, s2, N2, 0)
+    ok(lib, lib.drhip_softmax_ex_f32(None, ctypes.byref(d2), prob2, N2, None))
+    assert np.array_equal(dev.get(prob2, (N2,)), wantp)
+    # argument checks
+    bad = DeferredVec(q1.value, b1d.value, s1, N1 + 1, 1)
+    assert lib.drhip_fc_ex_f32(None, ctypes.byref(bad), W2d, b2d, y2b, q2, N1, N2, 0, 0, None) == -1
+    assert lib.drhip_fc_ex_f32(xd, None, W1d, b1d, None, None, 64, 8, 0, 1, None) == -1        # unsplit layers cannot defer
+
+
 def test_softmax(lib, dev, oracle):
     for n, scale in [(1000, 3.0), (10, 1.0), (5000, 5.0), (1, 1.0)]:
         x = rnd(n, scale=scale)
