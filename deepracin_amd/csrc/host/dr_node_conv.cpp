@@ -6,6 +6,8 @@
 // weights in the layout that kernel streams best, compute() enqueues through drhip_*.
 #include "dr_internal.hpp"
 
+#include <vector>
+
 using namespace dr;
 
 namespace {
@@ -90,13 +92,25 @@ gboolean conv_schedule(dR_Graph* net, dR_Node* node) {
 
 gboolean conv_create_kernel(dR_Graph*, dR_Node*) { return TRUE; }   // kernels are built into the library
 
+// Output channels the node's launch produces: its own plus those of an absorbed 1x1 sibling.
+inline int launch_channels(const dR_Conv2d_Data* c) {
+    return c->shape.s3 + (c->drAbsorbed1x1 ? conv_of(c->drAbsorbed1x1)->shape.s3 : 0);
+}
+inline bool launch_has_bias(const dR_Conv2d_Data* c) {
+    return c->useBias || (c->drAbsorbed1x1 && conv_of(c->drAbsorbed1x1)->useBias);
+}
+
 gboolean conv_allocate(dR_Graph* net, dR_Node* node) {
     dR_Conv2d_Data* c = conv_of(node);
+    if (c->drAbsorbedBy) return TRUE;           // the 3x3 sibling carries this node's filters and bias
     const bool wino = c->algo == drConvWinograd;
-    const int n = wino ? (int)drhip_conv3x3_winograd_filter_floats(c->shape.s2, c->shape.s3) : weight_count(c);
+    const int O = launch_channels(c);
+    if (c->drAbsorbed1x1)                       // the joint layer is wider than the one schedule() saw
+        c->variant = drhip_conv3x3_winograd_pick_variant(c->ishape.s0, c->ishape.s1, c->shape.s2, O);
+    const int n = wino ? (int)drhip_conv3x3_winograd_filter_floats(c->shape.s2, O) : weight_count(c);
     gboolean ok = dR_createFloatBuffer(net, &c->weightsBuf, n, CL_MEM_READ_ONLY);
-    if (c->useBias) ok = ok && dR_createFloatBuffer(net, &c->biasBuf, c->shape.s3, CL_MEM_READ_ONLY);
-    const size_t ws = wino ? drhip_conv3x3_winograd_workspace_floats(c->ishape.s0, c->ishape.s1, c->shape.s2, c->shape.s3, c->variant) : 0;
+    if (launch_has_bias(c)) ok = ok && dR_createFloatBuffer(net, &c->biasBuf, O, CL_MEM_READ_ONLY);
+    const size_t ws = wino ? drhip_conv3x3_winograd_workspace_floats(c->ishape.s0, c->ishape.s1, c->shape.s2, O, c->variant) : 0;
     if (ws > 0) ok = ok && dR_createFloatBuffer(net, &c->workspaceBuf, (gint)ws, CL_MEM_READ_WRITE);   // split-K partial tiles
     return ok;
 }
@@ -104,21 +118,42 @@ gboolean conv_allocate(dR_Graph* net, dR_Node* node) {
 gboolean conv_fill(dR_Graph* net, dR_Node* node) {
     dR_Conv2d_Data* c = conv_of(node);
     if (!c->hasVariables) { say("Conv2d Layer %d has no weights: call dR_Conv2d_setVariables first! \n", node->layerID); return FALSE; }
-    const size_t rawBytes = (size_t)weight_count(c) * sizeof(float);
+    if (c->drAbsorbedBy) return TRUE;
     gboolean ok = TRUE;
     if (c->algo == drConvWinograd) {
-        // raw weights go up once, U = G g G^T is produced on the device, the raw copy is dropped
+        // raw weights go up once, U = G g G^T is produced on the device, the raw copy is dropped.
+        // With an absorbed 1x1 sibling the joint filter bank is [I][O1 + O3][3][3]: the sibling's
+        // channels first (they sit just below this node's in the concat), centre tap only.
+        const dR_Conv2d_Data* a = c->drAbsorbed1x1 ? conv_of(c->drAbsorbed1x1) : NULL;
+        if (a && !a->hasVariables) { say("Conv2d Layer %d has no weights: call dR_Conv2d_setVariables first! \n", c->drAbsorbed1x1->layerID); return FALSE; }
+        const int I = c->shape.s2, O3 = c->shape.s3, O1 = a ? a->shape.s3 : 0, O = O1 + O3;
+        std::vector<float> joint;
+        const float* host = c->weights;
+        if (a) {
+            joint.assign((size_t)I * O * 9, 0.0f);
+            for (int i = 0; i < I; ++i) {
+                for (int o = 0; o < O1; ++o) joint[((size_t)i * O + o) * 9 + 4] = a->weights[(size_t)i * O1 + o];
+                memcpy(&joint[((size_t)i * O + O1) * 9], &c->weights[(size_t)i * O3 * 9], (size_t)O3 * 9 * sizeof(float));
+            }
+            host = joint.data();
+        }
+        const size_t rawBytes = (size_t)I * O * 9 * sizeof(float);
         cl_mem raw = NULL;
-        if (!dR_createFloatBuffer(net, &raw, weight_count(c), CL_MEM_READ_ONLY)) return FALSE;
-        ok = dR_uploadArray(net, (gchar*)"", c->weights, 0, rawBytes, raw);
-        if (ok) ok = !device_failed(net, drhip_winograd_filter_transform_f32((const float*)raw, (float*)c->weightsBuf,
-                                                                              c->shape.s2, c->shape.s3, stream_of(net)),
+        if (!dR_createFloatBuffer(net, &raw, I * O * 9, CL_MEM_READ_ONLY)) return FALSE;
+        ok = dR_uploadArray(net, (gchar*)"", (void*)host, 0, rawBytes, raw);
+        if (ok) ok = !device_failed(net, drhip_winograd_filter_transform_f32((const float*)raw, (float*)c->weightsBuf, I, O, stream_of(net)),
                                     "winograd filter transform");
         if (ok) ok = !device_failed(net, drhip_stream_sync(stream_of(net)), "winograd filter transform (sync)");
         dR_clMemoryBufferCleanup(net, raw);
         net->clConfig->memConsumptionGPU -= (glong)rawBytes;
+        if (ok && a && launch_has_bias(c)) {
+            std::vector<float> bias((size_t)O, 0.0f);
+            if (a->useBias) memcpy(bias.data(), a->biases, (size_t)O1 * sizeof(float));
+            if (c->useBias) memcpy(bias.data() + O1, c->biases, (size_t)O3 * sizeof(float));
+            return dR_uploadArray(net, (gchar*)"", bias.data(), 0, (size_t)O * sizeof(float), c->biasBuf);
+        }
     } else {
-        ok = dR_uploadArray(net, (gchar*)"", c->weights, 0, rawBytes, c->weightsBuf);
+        ok = dR_uploadArray(net, (gchar*)"", c->weights, 0, (size_t)weight_count(c) * sizeof(float), c->weightsBuf);
     }
     if (ok && c->useBias) ok = dR_uploadArray(net, (gchar*)"", c->biases, 0, (size_t)c->shape.s3 * sizeof(float), c->biasBuf);
     return ok;
@@ -126,12 +161,15 @@ gboolean conv_fill(dR_Graph* net, dR_Node* node) {
 
 gboolean conv_compute(dR_Graph* net, dR_Node* node) {
     dR_Conv2d_Data* c = conv_of(node);
+    if (c->drAbsorbedBy) return TRUE;           // computed by the 3x3 sibling's launch
     dR_Node* src = first_input(node);
     const float* in = dev_out(src);
-    float* out = dev_out(node);         // with drFusedPool this is the pooling node's buffer
+    // with drFusedPool this is the pooling node's buffer; with an absorbed 1x1 sibling the launch
+    // starts at that sibling's channels, which lie directly below this node's in the concat buffer
+    float* out = c->drAbsorbed1x1 ? dev_out(c->drAbsorbed1x1) : dev_out(node);
     const float* w = (const float*)c->weightsBuf;
-    const float* b = c->useBias ? (const float*)c->biasBuf : NULL;
-    const int W = c->ishape.s0, H = c->ishape.s1, I = c->shape.s2, O = c->shape.s3;
+    const float* b = launch_has_bias(c) ? (const float*)c->biasBuf : NULL;
+    const int W = c->ishape.s0, H = c->ishape.s1, I = c->shape.s2, O = launch_channels(c);
     const int relu = c->activation == tReLU;
     int rc;
     switch (c->algo) {
@@ -154,7 +192,7 @@ gboolean conv_compute(dR_Graph* net, dR_Node* node) {
 gboolean conv_cleanup_buffers(dR_Graph* net, dR_Node* node) {
     dR_Conv2d_Data* c = conv_of(node);
     gboolean ok = dR_clMemoryBufferCleanup(net, c->weightsBuf);
-    if (c->useBias) ok = dR_clMemoryBufferCleanup(net, c->biasBuf) && ok;
+    ok = dR_clMemoryBufferCleanup(net, c->biasBuf) && ok;
     ok = dR_clMemoryBufferCleanup(net, c->workspaceBuf) && ok;
     c->weightsBuf = c->biasBuf = c->workspaceBuf = NULL;
     return ok;

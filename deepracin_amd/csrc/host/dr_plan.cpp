@@ -50,6 +50,23 @@ bool concat_can_fuse(const dR_Node* c) {
     return !ins.empty();
 }
 
+// The expand pair of a fire module: a 1x1 and a 3x3 convolution of the same tensor whose outputs sit
+// next to each other in a fused channel concat.  A 1x1 filter is a 3x3 filter with only its centre
+// tap, so both become ONE Winograd launch over the joint output channels (DR_FUSE_EXPAND=0 keeps
+// them apart).  The 1x1 outputs then come out of the Winograd transforms instead of the plain
+// dot product: same function, fp32 rounding differs at the 1e-6 level.
+bool expand_pair(const dR_Node* a, const dR_Node* b) {
+    const char* env = getenv("DR_FUSE_EXPAND");
+    if (env && strcmp(env, "0") == 0) return false;
+    if (a->type != tConv2d || b->type != tConv2d) return false;
+    const dR_Conv2d_Data* ca = (const dR_Conv2d_Data*)a->layer;
+    const dR_Conv2d_Data* cb = (const dR_Conv2d_Data*)b->layer;
+    if (ca->algo != drConv1x1Gemm || cb->algo != drConvWinograd) return false;
+    if (ca->activation != cb->activation || ca->shape.s2 != cb->shape.s2) return false;
+    std::vector<dR_Node*> ia = nodes_of(a->previous_layers), ib = nodes_of(b->previous_layers);
+    return ia.size() == 1 && ib.size() == 1 && ia[0] == ib[0];
+}
+
 // A 2x2 / stride-2 max pool directly behind a Winograd convolution: every 2x2 output tile of the
 // convolution is one pooling window, so the convolution's epilogue can store the maximum and the
 // full-resolution tensor never exists.  Only when nobody else wants that tensor.
@@ -200,6 +217,8 @@ gboolean dR_planBuffers(dR_Graph* net) {
         else continue;
         fd->drDeferReduce = TRUE;
     }
+    for (dR_Node* n : sched)
+        if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drAbsorbed1x1 = ((dR_Conv2d_Data*)n->layer)->drAbsorbedBy = nullptr;
     for (dR_Node* n : sched) {
         if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drFusedPool = FALSE;
         if (n->type == tPooling) {
@@ -212,10 +231,16 @@ gboolean dR_planBuffers(dR_Graph* net) {
         cd->drFused = concat_can_fuse(n);
         if (!cd->drFused) continue;
         int off = 0;
-        for (dR_Node* p : nodes_of(n->previous_layers)) {
+        std::vector<dR_Node*> ins = nodes_of(n->previous_layers);
+        for (dR_Node* p : ins) {
             parent[p] = std::make_pair(n, off);
             off += p->oshape.s0 * p->oshape.s1 * p->oshape.s2;
         }
+        for (size_t k = 0; k + 1 < ins.size(); ++k)
+            if (expand_pair(ins[k], ins[k + 1]) && !((dR_Conv2d_Data*)ins[k]->layer)->drAbsorbedBy) {
+                ((dR_Conv2d_Data*)ins[k]->layer)->drAbsorbedBy = ins[k + 1];
+                ((dR_Conv2d_Data*)ins[k + 1]->layer)->drAbsorbed1x1 = ins[k];
+            }
     }
     auto root_of = [&](dR_Node* n, int* offset) {
         int off = 0;

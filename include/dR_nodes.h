@@ -43,6 +43,9 @@ struct dR_Conv2d_Data {
     gint                variant;        /* tile configuration id understood by the drhip_* launcher */
     gint                winogradn;      /* always 2: F(2x2,3x3) */
     cl_mem              workspaceBuf;   /* split-K scratch of the Winograd kernel, NULL when the layer is not split */
+    dR_Node*            drAbsorbed1x1;  /* set by the buffer planner on a Winograd node: the 1x1 sibling (same input, the channels
+                                           just below this node's in a fused concat) whose filters ride along as centre taps */
+    dR_Node*            drAbsorbedBy;   /* set on that 1x1 sibling: its compute() launches nothing */
     gboolean            drFusedPool;    /* set by the buffer planner: the node's only consumer is a 2x2/2 max pool and
                                            this node writes the pooled tensor straight into that node's buffer */
 };
