@@ -51,14 +51,17 @@ conv_direct_kernel(const float* __restrict__ in, const float* __restrict__ w, co
         for (int e = tid; e < cc * patchN; e += kDirThreads) {
             const int c = e / patchN, r = e % patchN;
             const int gx = px0 + r % patchW, gy = py0 + r / patchW;
-            float v = 0.0f;
-            if (gx >= 0 && gx < W && gy >= 0 && gy < H) v = in[(size_t)(c0 + c) * H * W + (size_t)gy * W + gx];
-            patch[e] = v;
+            // unconditional load from the clamped position, zero padding by select: loads under a
+            // per-lane branch are waited for one by one
+            const bool inside = gx >= 0 && gx < W && gy >= 0 && gy < H;
+            const float v = in[(size_t)(c0 + c) * H * W + (size_t)min(max(gy, 0), H - 1) * W + min(max(gx, 0), W - 1)];
+            patch[e] = inside ? v : 0.0f;
         }
         for (int e = tid; e < cc * taps * OCT; e += kDirThreads) {
             const int oc = e % OCT, tap = (e / OCT) % taps, c = e / (OCT * taps);
             const int o = o0 + oc;
-            filt[e] = (o < O) ? w[((size_t)(c0 + c) * O + o) * taps + tap] : 0.0f;
+            const float f = w[((size_t)(c0 + c) * O + min(o, O - 1)) * taps + tap];
+            filt[e] = (o < O) ? f : 0.0f;
         }
         __syncthreads();
         for (int c = 0; c < cc; ++c) {
@@ -92,6 +95,65 @@ conv_direct_kernel(const float* __restrict__ in, const float* __restrict__ w, co
                 float v = acc[k] + (bias ? bias[o] : 0.0f);
                 if (relu) v = fmaxf(v, 0.0f);
                 out[(size_t)o * Ho * Wo + (size_t)yo * Wo + xo] = v;
+            }
+        }
+    }
+}
+
+// First layers (I <= 4, e.g. RGB): too little work per channel to pay for staging anything in LDS.
+// One lane = one output pixel x OCT channels; its kw*kh*I input samples come straight from global
+// memory (unconditional loads from clamped positions, zero padding by select; neighbours share
+// cache lines), and the filters are wave-uniform, so the compiler fetches them with scalar loads
+// and the FMAs take them from SGPRs.
+template <int OCT, int KW, int KH>
+__global__ void __launch_bounds__(kDirThreads)
+conv_direct_fewc_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
+                        float* __restrict__ out, int W, int H, int I, int O, int Wo, int Ho,
+                        int sx, int sy, int tilesX, int relu) {
+    constexpr int taps = KW * KH;
+    const int tid = threadIdx.x, tx = tid % kDirTile, ty = tid / kDirTile;
+    const int tileX = blockIdx.x % tilesX, tileY = blockIdx.x / tilesX;
+    const int o0 = blockIdx.y * OCT;
+    const int xo = tileX * kDirTile + tx, yo = tileY * kDirTile + ty;
+    const int cx = min(xo, Wo - 1) * sx - KW / 2, cy = min(yo, Ho - 1) * sy - KH / 2;   // window origin (clamped lanes recompute a valid pixel)
+
+    float acc[OCT];
+#pragma unroll
+    for (int k = 0; k < OCT; ++k) acc[k] = 0.0f;
+
+    // all samples of all (up to 4) channels first: one memory latency for the whole lane
+    float v[4][taps];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const float* pc = in + (size_t)min(c, I - 1) * H * W;
+#pragma unroll
+        for (int j = 0; j < KH; ++j)
+#pragma unroll
+            for (int i = 0; i < KW; ++i) {
+                const int gx = cx + i, gy = cy + j;
+                const float raw = pc[(size_t)min(max(gy, 0), H - 1) * W + min(max(gx, 0), W - 1)];
+                v[c][j * KW + i] = (c < I && gx >= 0 && gx < W && gy >= 0 && gy < H) ? raw : 0.0f;
+            }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        if (c < I) {                                 // uniform
+#pragma unroll
+            for (int k = 0; k < OCT; ++k) {
+                const float* fk = w + ((size_t)c * O + min(o0 + k, O - 1)) * taps;     // wave-uniform address
+#pragma unroll
+                for (int t = 0; t < taps; ++t) acc[k] = fmaf(v[c][t], fk[t], acc[k]);
+            }
+        }
+    }
+    if (xo < Wo && yo < Ho) {
+#pragma unroll
+        for (int k = 0; k < OCT; ++k) {
+            const int o = o0 + k;
+            if (o < O) {
+                float r = acc[k] + (bias ? bias[o] : 0.0f);
+                if (relu) r = fmaxf(r, 0.0f);
+                out[(size_t)o * Ho * Wo + (size_t)yo * Wo + xo] = r;
             }
         }
     }
@@ -131,6 +193,18 @@ extern "C" int drhip_conv2d_direct_f32(const float* in, const float* w, const fl
     DRHIP_REQUIRE(W / strideX > 0 && H / strideY > 0, "drhip_conv2d_direct_f32: output is empty");
     DRHIP_REQUIRE((long long)W * H * I < (1ll << 31) && (long long)(W / strideX) * (H / strideY) * O < (1ll << 31),
                   "drhip_conv2d_direct_f32: tensor too large");
+    hipStream_t s0 = as_stream(stream);
+    if (I <= 4 && kw == 3 && kh == 3) {
+        const int Wo = W / strideX, Ho = H / strideY;
+        const int tilesX = ceil_div(Wo, kDirTile), tilesY = ceil_div(Ho, kDirTile);
+        if (O >= 8)
+            launch((conv_direct_fewc_kernel<8, 3, 3>), dim3(tilesX * tilesY, ceil_div(O, 8)), dim3(kDirThreads), 0, s0,
+                   in, w, bias, out, W, H, I, O, Wo, Ho, strideX, strideY, tilesX, relu);
+        else
+            launch((conv_direct_fewc_kernel<4, 3, 3>), dim3(tilesX * tilesY, ceil_div(O, 4)), dim3(kDirThreads), 0, s0,
+                   in, w, bias, out, W, H, I, O, Wo, Ho, strideX, strideY, tilesX, relu);
+        return launched("conv_direct_fewc_kernel");
+    }
     // Few output channels per lane when the tile count alone cannot fill the CUs.
     const int tiles = ceil_div(W / strideX, kDirTile) * ceil_div(H / strideY, kDirTile);
     hipStream_t s = as_stream(stream);

@@ -68,6 +68,7 @@ def ok(lib, rc):
     (56, 56, 64, 64, 3, 1),      # config 1, direct variant
     (224, 224, 3, 64, 3, 2),     # SqueezeNet conv1
     (17, 13, 5, 7, 3, 1), (20, 18, 4, 20, 5, 1), (33, 31, 3, 9, 3, 2), (16, 16, 2, 3, 7, 3), (9, 9, 1, 1, 1, 2),
+    (37, 21, 4, 33, 3, 1), (8, 5, 1, 16, 3, 3), (2, 2, 3, 2, 3, 1),     # I <= 4 with a 3x3 filter: the no-LDS first-layer kernel
 ])
 def test_conv_direct(lib, dev, oracle, W, H, I, O, k, s):
     x, w, b = np.abs(rnd(I, H, W)), rnd(I, O, k, k, scale=np.sqrt(2.0 / (k * k * I))), rnd(O, scale=0.01)
