@@ -49,6 +49,7 @@ struct FcPlan { int vec, cbw, panels, slices, rowsPerSlice; };
 static FcPlan fc_plan(int K, int N) {
     FcPlan p;
     p.vec = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+    while (p.vec > 1 && ceil_div(N, kWave * p.vec) < 16) p.vec /= 2;    // narrow matrices (N = 1000): more, narrower panels
     p.cbw = kWave * p.vec;
     p.panels = ceil_div(N, p.cbw);
     const int target = 4 * num_cu();                 // workgroups wanted in flight
