@@ -109,14 +109,16 @@ __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, 
 //
 //   * wave w (0..3) of a 256-lane workgroup owns the transform positions xi = 4w..4w+3, i.e. row w
 //     of B^T d B.  That row needs only TWO rows of the 4x4 input window (row w combined with row 2
-//     or 1), so a lane loads 8 floats and spends 8 adds per (tile, channel) - and the four results
-//     are exactly the B operands (lane -> tile lane%32, k -> channel parity lane/32) of that wave's
-//     own MFMAs.  V never goes through LDS and the waves of a workgroup never synchronise inside
-//     the channel loop.
-//   * the window samples are fetched with raw buffer loads whose resource covers the channels from
-//     the current one to the end of the tensor: samples outside the image carry an offset beyond
+//     or 1), so a lane loads two rows of 4 floats and spends 8 adds per (tile, channel) - and the
+//     four results are exactly the B operands (lane -> tile lane%32, k -> channel parity lane/32)
+//     of that wave's own MFMAs.  V never goes through LDS and the waves of a workgroup never
+//     synchronise inside the channel loop.
+//   * a window row is ONE 16-byte raw buffer load (four dword loads per row kept the CU's single
+//     address unit busier than the matrix cores).  The resource covers the channels from the
+//     current one to the end of the tensor: rows above or below the image carry an offset beyond
 //     the resource, channels past the last one see a resource of size zero, and the hardware
-//     returns 0.0 for both - zero padding and ragged channel counts cost no instruction.
+//     returns 0.0 for both - vertical padding and ragged channel counts cost no instruction.
+//     Samples left or right of the image are zeroed by selects after the two rows are combined.
 //   * all addresses are a per-lane byte offset computed once plus scalar (SGPR) bases.
 //   * operands of the next stage are loaded into the registers the current stage has just
 //     finished with (input rows after their transform, filters after the MFMAs of their xi pair),
