@@ -134,6 +134,7 @@ def load_library(path=None):
         "dR_Concat": (vp, [vp, POINTER(vp), c_int, c_int]),
         "dR_Slice": (vp, [vp, vp, POINTER(Shape4), POINTER(Shape4)]),
         "dR_ElemWise1Operation": (vp, [vp, vp, c_int, c_float]),
+        "dR_Normalization": (vp, [vp, vp, c_int, c_float, c_float]),
         # device layer
         "drhip_init": (c_int, [c_int, POINTER(DeviceInfo)]),
         "drhip_last_error": (c_char_p, []),
@@ -156,6 +157,8 @@ def load_library(path=None):
         "drhip_fc_slices": (c_int, [c_int, c_int]),
         "drhip_fc_ex_f32": (c_int, [vp, vp, vp, vp, vp, vp, c_int, c_int, c_int, c_int, vp]),
         "drhip_softmax_ex_f32": (c_int, [vp, vp, vp, c_int, vp]),
+        "drhip_normalize_scratch_floats": (c_size_t, [c_size_t]),
+        "drhip_normalize_f32": (c_int, [vp, vp, c_size_t, c_int, c_float, c_float, vp, vp]),
         "drhip_timing_begin": (c_int, []),
         "drhip_timing_count": (c_int, []),
         "drhip_timing_end": (c_int, [POINTER(c_float), c_int, POINTER(c_int)]),
@@ -449,6 +452,17 @@ def Pooling(input_node, pooling_type, shape, stride):
 def Softmax(input_node):
     g = input_node.graph
     return Node(g.lib.dR_Softmax(g.ptr, input_node.ptr), g, "Softmax", [])
+
+
+norm_dict = {"target_mean": 0, "target_dev": 1, "target_mean_dev": 2}
+
+
+def Normalization(input_node, normalization_type, target_mean=0.0, target_dev=1.0):
+    """Reference wrapper :889-898; normalization_type is a key of norm_dict (or its number)."""
+    g = input_node.graph
+    kind = norm_dict.get(normalization_type, normalization_type)
+    return Node(g.lib.dR_Normalization(g.ptr, input_node.ptr, int(kind), c_float(target_mean), c_float(target_dev)), g,
+                "Normalization", [kind, target_mean, target_dev])
 
 
 def Slice(input_node, origin, shape):

@@ -10,6 +10,7 @@ index.  The same spec is (a) turned into a deepRacin graph through the C API by 
     {"op": "fc", "in": i, "w": [K,N] f32 (k counts the input in [H][W][C] order), "b": [N] | None, "relu": bool}
     {"op": "softmax", "in": i}
     {"op": "concat", "ins": [i, j, ...], "dim": 2}
+    {"op": "norm", "in": i, "kind": 0 mean | 1 deviation | 2 both, "mean": target, "dev": target}
 
 Random numbers: numpy PCG64 from one seed, one sub-stream per tensor.  Tensors are drawn in the
 logical interface layout (HWC images, HWIO filters) and converted to the C API layouts exactly as
@@ -98,11 +99,16 @@ def vgg_conv3_block(seed=0, size=56, cin=128, cout=256):
     return spec, {0: image_input(st, size, size, cin)}, [4]
 
 
-def squeezenet11(seed=0, size=224, classes=1000):
-    """Config 4: SqueezeNet v1.1 topology, random He-normal weights, per-image normalised input."""
+def squeezenet11(seed=0, size=224, classes=1000, normalise_in_graph=False):
+    """Config 4: SqueezeNet v1.1 topology, random He-normal weights, per-image normalised input.
+
+    normalise_in_graph: feed the raw U[0,255) image and let a Normalization node (mean 0, deviation 1)
+    in front of conv1 do what the generator otherwise does on the host."""
     st = _Streams(seed)
     spec = [{"op": "feed", "shape": (size, size, 3)}]
-    spec.append(_conv(st, 0, 3, 3, 64, stride=2))
+    if normalise_in_graph:
+        spec.append({"op": "norm", "in": 0, "kind": 2, "mean": 0.0, "dev": 1.0})
+    spec.append(_conv(st, len(spec) - 1, 3, 3, 64, stride=2))
     spec.append(_maxpool(len(spec) - 1, 3, 2)); cur, cin = len(spec) - 1, 64
     plan = [(16, 64), (16, 64), "pool", (32, 128), (32, 128), "pool", (48, 192), (48, 192), (64, 256), (64, 256)]
     for item in plan:
@@ -116,7 +122,7 @@ def squeezenet11(seed=0, size=224, classes=1000):
         fin = -(-fin // 2)
     spec.append({"op": "pool", "in": cur, "window": (fin, fin, 1), "stride": (fin, fin, 1), "kind": 1}); cur = len(spec) - 1
     spec.append({"op": "softmax", "in": cur})
-    return spec, {0: image_input(st, size, size, 3, scale=255.0, normalise=True)}, [len(spec) - 1, len(spec) - 2]
+    return spec, {0: image_input(st, size, size, 3, scale=255.0, normalise=not normalise_in_graph)}, [len(spec) - 1, len(spec) - 2]
 
 
 def vgg16(seed=0, size=224, classes=1000, fc_width=4096):
@@ -174,6 +180,8 @@ def build_graph(graph, spec, outputs):
         elif op == "slice":
             o, s = dr.Shape4(*n["origin"], 0), dr.Shape4(*n["shape"], 0)
             node = dr.Node(lib.dR_Slice(graph.ptr, nodes[n["in"]].ptr, dr.pointer(o), dr.pointer(s)), graph, "Slice", [])
+        elif op == "norm":
+            node = dr.Normalization(nodes[n["in"]], n["kind"], n["mean"], n["dev"])
         elif op == "scalar":
             node = dr.Node(lib.dR_ElemWise1Operation(graph.ptr, nodes[n["in"]].ptr, n["kind"], dr.c_float(n["value"])), graph, "ElemWise1Op", [])
         else:

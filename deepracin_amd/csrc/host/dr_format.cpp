@@ -75,11 +75,12 @@ const Kind kKinds[] = {
     { "Slice",          dR_slice_parseAppendNode,        1, 1 },
     { "Concat",         dR_concat_parseAppendNode,       2, 256 },
     { "ElemWise1Op",    dR_elemwise1op_parseAppendNode,  1, 1 },
+    { "Normalization",  dR_norm_parseAppendNode,         1, 1 },
     { "DataFeedNode",   dR_datafeednode_parseAppendNode, 0, 0 },
 };
 
 // Node kinds of the reference that exist in graph.dr files but lie outside the CNN layer path.
-const char* const kForeign[] = { "PPFilter", "MaskDependentFilter", "LabelCreation", "Normalization", "Upscaling",
+const char* const kForeign[] = { "PPFilter", "MaskDependentFilter", "LabelCreation", "Upscaling",
                                  "RGB2Gray", "ResolveRoI", "CropOrPad", "ElemWise2Op" };
 
 }  // namespace

@@ -82,4 +82,5 @@ dR_Node* dR_softmax_parseAppendNode(dR_Graph*, dR_Node**, gint, gchar**, gint, g
 dR_Node* dR_concat_parseAppendNode(dR_Graph*, dR_Node**, gint, gchar**, gint, gfloat**, gint);
 dR_Node* dR_slice_parseAppendNode(dR_Graph*, dR_Node**, gint, gchar**, gint, gfloat**, gint);
 dR_Node* dR_elemwise1op_parseAppendNode(dR_Graph*, dR_Node**, gint, gchar**, gint, gfloat**, gint);
+dR_Node* dR_norm_parseAppendNode(dR_Graph*, dR_Node**, gint, gchar**, gint, gfloat**, gint);
 }

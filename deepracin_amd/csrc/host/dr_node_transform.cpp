@@ -1,6 +1,6 @@
 // Concat, Slice and element-wise scalar nodes (host side).
 // Contracts: reference src/dR_nodes_transform.c:8-232 (Slice), :238-569 (Concat),
-// src/dR_nodes_math.c:259-527 (ElemWise1Op).
+// src/dR_nodes_math.c:259-527 (ElemWise1Op), src/dR_nodes_misc.c:1046-1546 (Normalization).
 #include "dr_internal.hpp"
 
 using namespace dr;
@@ -171,9 +171,94 @@ gchar* ew_print(dR_Node* node) {
     return fmt_dup("Element-wise 1-operation node: %d\n Operation: %s\n Scalar: %f\n", node->layerID, ops[(unsigned)e->op % 9], e->scalar);
 }
 
+// ================================ Normalization ==================================================
+
+inline dR_Normalization_Data* norm_of(dR_Node* n) { return (dR_Normalization_Data*)n->layer; }
+
+gboolean norm_propagate(dR_Graph* net, dR_Node* node) {
+    if (node->previous_layers->length != 1 && verbose(net))
+        say("Normalization Layer with id %d has %d inputs but needs 1!\n", node->layerID, node->previous_layers->length);
+    dR_Node* in = first_input(node);
+    if (!in) return FALSE;
+    norm_of(node)->ishape = in->oshape;
+    node->oshape = in->oshape;
+    return TRUE;
+}
+
+gboolean norm_allocate(dR_Graph* net, dR_Node* node) {
+    dR_Normalization_Data* d = norm_of(node);
+    return dR_createFloatBuffer(net, &d->tempFloatBuffer1, (gint)drhip_normalize_scratch_floats((size_t)out_volume(node)), CL_MEM_READ_WRITE);
+}
+
+gboolean norm_compute(dR_Graph* net, dR_Node* node) {
+    dR_Normalization_Data* d = norm_of(node);
+    int rc = drhip_normalize_f32(dev_out(first_input(node)), dev_out(node), (size_t)out_volume(node), (int)d->type,
+                                 d->targetMean, d->targetDev, (float*)d->tempFloatBuffer1, stream_of(net));
+    return !device_failed(net, rc, "deepRACIN:normalization");
+}
+
+gboolean norm_cleanup_buffers(dR_Graph* net, dR_Node* node) {
+    dR_Normalization_Data* d = norm_of(node);
+    gboolean ok = dR_clMemoryBufferCleanup(net, d->tempFloatBuffer1);
+    d->tempFloatBuffer1 = NULL;
+    return ok;
+}
+
+gchar* norm_serialize(dR_Node* node, gchar* params[], gint* numParams, gfloat*[], gint[], gint* numVariables) {
+    dR_Normalization_Data* d = norm_of(node);
+    if (*numParams < 3) { say("SerializeNode needs space for 3 parameters and 0 variables!\n"); return NULL; }
+    params[0] = fmt_dup("%d", (int)d->type);
+    params[1] = fmt_dup("%f", d->targetMean);
+    params[2] = fmt_dup("%f", d->targetDev);
+    *numParams = 3;
+    *numVariables = 0;
+    return (gchar*)"Normalization";
+}
+
+gchar* norm_print(dR_Node* node) {
+    dR_Normalization_Data* d = norm_of(node);
+    static const char* kinds[] = { "Mean", "Deviation", "Mean and deviation" };
+    return fmt_dup("Normalization Layer: %d\n Type: %s\n Target mean: %f\n Target deviation: %f\n", node->layerID,
+                   kinds[(unsigned)d->type % 3], d->targetMean, d->targetDev);
+}
+
 }  // namespace
 
 extern "C" {
+
+dR_Node* dR_Normalization(dR_Graph* net, dR_Node* inputLayer, dR_NormalizationType type, gfloat targetMean, gfloat targetDev) {
+    dR_Normalization_Data* d = zalloc<dR_Normalization_Data>();
+    dR_Node* n = zalloc<dR_Node>();
+    d->type = type;
+    d->targetMean = targetMean;
+    d->targetDev = targetDev;
+    n->layer = d;
+    n->type = tNormalization;
+    n->compute = norm_compute;
+    n->schedule = nothing;
+    n->propagateShape = norm_propagate;
+    n->getRequiredOutputBufferSize = out_volume;
+    n->createKernel = nothing;
+    n->allocateBuffers = norm_allocate;
+    n->fillBuffers = nothing;
+    n->cleanupBuffers = norm_cleanup_buffers;
+    n->cleanupLayer = free_layer;
+    n->serializeNode = norm_serialize;
+    n->parseAppendNode = dR_norm_parseAppendNode;
+    n->printLayer = norm_print;
+    link_single_input(n, inputLayer, "Normalization Layer");
+    dR_appendLayer(net, n);
+    return n;
+}
+
+dR_Node* dR_norm_parseAppendNode(dR_Graph* net, dR_Node** iNodes, gint numINodes, gchar** params, gint numParams,
+                                 gfloat**, gint numVariables) {
+    if (numINodes != 1) { say("Parsing Error: Normalization Node needs 1 InputNodes but got %d!\n", numINodes); return NULL; }
+    if (numParams != 3 || numVariables != 0) { say("Parsing Error: Normalization Node needs 3 Parameters and 0 Variables!\n"); return NULL; }
+    const int type = atoi(params[0]);
+    if (type < 0 || type > 2) { say("Parsing Error: Normalization type %d unknown!\n", type); return NULL; }
+    return dR_Normalization(net, iNodes[0], (dR_NormalizationType)type, (gfloat)atof(params[1]), (gfloat)atof(params[2]));
+}
 
 dR_Node* dR_Concat(dR_Graph* net, dR_Node** inputNodes, gint n, gint concatDim) {
     dR_Concat_Data* c = zalloc<dR_Concat_Data>();

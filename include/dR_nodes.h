@@ -162,6 +162,29 @@ struct dR_ElemWise1Op_Data {
 dR_Node* dR_ElemWise1Operation(dR_Graph* net, dR_Node* inputNode, dR_ElemWise1OperationType op,
                                gfloat scalar);
 
+/* ================================ normalization =============================================== */
+
+/* Same numbering as the reference (include/dR_nodes_misc.h:268-272). */
+enum dR_NormalizationType { tNormMean, tNormDev, tNormMeanDev };
+typedef enum dR_NormalizationType dR_NormalizationType;
+
+typedef struct dR_Normalization_Data dR_Normalization_Data;
+struct dR_Normalization_Data {
+    dR_Shape3               ishape;
+    dR_NormalizationType    type;
+    gfloat                  targetMean;
+    gfloat                  targetDev;
+    cl_mem                  tempFloatBuffer1;   /* per-workgroup partial sums of both reductions */
+    cl_mem                  tempFloatBuffer2;   /* unused placeholder (the reference ping-pongs between two) */
+};
+
+/* Shift and/or scale the whole input tensor to a target mean / standard deviation taken over all
+ * W*H*C elements (population deviation about the mean): tNormMean y = x + (targetMean - mean),
+ * tNormDev y = x * (targetDev / dev), tNormMeanDev both (reference src/dR_nodes_misc.c:1051-1446;
+ * graph.dr: "Normalization", params `type targetMean targetDev`). */
+dR_Node* dR_Normalization(dR_Graph* net, dR_Node* inputLayer, dR_NormalizationType type, gfloat targetMean,
+                          gfloat targetDev);
+
 #ifdef __cplusplus
 }
 #endif

@@ -182,6 +182,16 @@ int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, const float*
 /* dst[k_chw][n] = src[k_hwc][n] with k_hwc = (y*W + x)*C + z for k_chw = (z*H + y)*W + x. */
 int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, int H, int C, int N, void* stream);
 
+/* ---- normalization of a whole tensor (n elements) to a target mean and/or standard deviation:
+ * type 0: y = x + (targetMean - mean); 1: y = x * (targetDev / dev); 2: both, dev = population
+ * standard deviation about the mean.  Two (type 0) or three launches, no host round trip; `scratch`
+ * = drhip_normalize_scratch_floats(n) floats, no initialisation needed.  x and y 16-byte aligned.
+ * Replaces getAvg / getSumDev + blocking downloads + addScalar / mulScalar / addMulScalar
+ * (src/dR_nodes_misc.c:1163-1446, Kernels/dR_helper.cl:315-471, Kernels/dR_math.cl:100-144). */
+size_t drhip_normalize_scratch_floats(size_t n);
+int drhip_normalize_f32(const float* x, float* y, size_t n, int type, float targetMean, float targetDev,
+                        float* scratch, void* stream);
+
 /* ---- softmax: y = exp(x - max x) / sum exp(x - max x) over n elements, one workgroup, wavefront
  * shuffles.  Replaces computeExp + host-side sum + mulScalar (src/dR_nodes_math.c:620-678,
  * Kernels/dR_math.cl:216-227,295-305). */

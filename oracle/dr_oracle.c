@@ -19,6 +19,7 @@
  *   oracle_pool           torch max_pool2d/avg_pool2d(ceil_mode) on explicitly zero-padded input
  *   oracle_fc             fp64 GEMV with the HWC permutation, torch linear
  *   oracle_softmax        scipy.special.softmax
+ *   oracle_normalize      numpy mean / std in fp64 (closed form), constant-offset and scaling identities
  *   whole network         the reference's stored SqueezeNet v1.1 + tiger.png -> 292, puzzle.png -> 611
  *   stride > 1 conv       header formula only (include/dR_nodes_conv2d.h:47-54); the reference's
  *                         generated kernel ignores the stride, so no reference run could pin it.
@@ -313,5 +314,76 @@ DR_API void oracle_scalar_op(const float* x, float* y, size_t n, int op, float s
             case 7: y[i] = s; break;
             default: y[i] = powf(v, s); break;
         }
+    }
+}
+
+/* One pass of `getAvg` / `getSumDev` (Kernels/dR_helper.cl:315-471) over one channel plane of
+ * gW x gH values: work-groups of 16 x 8, each loads its values (0 outside the plane; `first`:
+ * (v - avg)^2 instead of v) and adds them with the halving tree lsum[lid] += lsum[lid + half],
+ * lid = ly*16 + lx.  One result per work-group, written row-major into `out`. */
+static void norm_tree_pass(const float* in, float* out, int gW, int gH, int first, float avg) {
+    const int ngx = (gW + 15) / 16, ngy = (gH + 7) / 8;
+    for (int gyb = 0; gyb < ngy; ++gyb)
+        for (int gxb = 0; gxb < ngx; ++gxb) {
+            float lsum[128];
+            for (int ly = 0; ly < 8; ++ly)
+                for (int lx = 0; lx < 16; ++lx) {
+                    const int gx = gxb * 16 + lx, gy = gyb * 8 + ly;
+                    float v = 0.0f;
+                    if (gx < gW && gy < gH) {
+                        v = in[gy * gW + gx];
+                        if (first) { const float d = v - avg; v = d * d; }
+                    }
+                    lsum[ly * 16 + lx] = v;
+                }
+            for (int half = 64; half >= 1; half >>= 1)
+                for (int lid = 0; lid < half; ++lid) lsum[lid] += lsum[lid + half];
+            out[gyb * ngx + gxb] = lsum[0];
+        }
+}
+
+/* Sum of one channel plane by repeated tree passes until one work-group is left
+ * (src/dR_nodes_misc.c:1206-1258, 1312-1368). */
+static float norm_plane_sum(const float* plane, int W, int H, int dev, float avg, float* t1, float* t2) {
+    const float* in = plane;
+    float* out = t1;
+    int gW = W, gH = H, first = dev;
+    for (;;) {
+        norm_tree_pass(in, out, gW, gH, first, avg);
+        const int ngx = (gW + 15) / 16, ngy = (gH + 7) / 8;
+        if (ngx * ngy == 1) return out[0];
+        in = out;
+        out = (out == t1) ? t2 : t1;
+        gW = ngx; gH = ngy; first = 0;
+    }
+}
+
+/* Normalization node, src/dR_nodes_misc.c:1163-1446: per-channel tree sums, a sequential host sum
+ * over the channels, mean = sum / (W*H*C); the same again for (x - mean)^2 and dev = sqrt(sum / n);
+ * then y = x + (targetMean - mean) [type 0], x * (1 / (dev / targetDev)) [type 1] or both [type 2]
+ * (`addScalar`, `mulScalar`, `addMulScalar`, Kernels/dR_math.cl:100-144).  The reference sizes its
+ * two scratch buffers for a single channel; this restatement gives every channel its own passes,
+ * which is what the kernel's indexing intends. */
+DR_API void oracle_normalize(const float* x, float* y, int W, int H, int C, int type, float targetMean, float targetDev) {
+    const size_t plane = (size_t)W * H, n = plane * C;
+    const int ng = ((W + 15) / 16) * ((H + 7) / 8);
+    float* t1 = (float*)malloc(sizeof(float) * (size_t)ng);
+    float* t2 = (float*)malloc(sizeof(float) * (size_t)ng);
+    float sum = 0.0f;
+    for (int c = 0; c < C; ++c) sum += norm_plane_sum(x + c * plane, W, H, 0, 0.0f, t1, t2);
+    const float gavg = sum / (float)n;
+    float gdev = 1.0f;
+    if (type == 1 || type == 2) {
+        sum = 0.0f;
+        for (int c = 0; c < C; ++c) sum += norm_plane_sum(x + c * plane, W, H, 1, gavg, t1, t2);
+        gdev = (float)sqrt(sum / (float)n);
+    }
+    free(t1);
+    free(t2);
+    const float add = -(gavg - targetMean), mul = 1.0f / (gdev / targetDev);
+    for (size_t i = 0; i < n; ++i) {
+        if (type == 0) y[i] = x[i] + add;
+        else if (type == 1) y[i] = x[i] * mul;
+        else y[i] = (x[i] + add) * mul;
     }
 }

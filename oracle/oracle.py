@@ -157,6 +157,23 @@ def scalar_op(x, op, s):
     return y
 
 
+def normalize(x, kind, target_mean=0.0, target_dev=1.0):
+    """Normalization node on x [C,H,W]: kind 0 mean, 1 deviation, 2 both (reference tree-sum order)."""
+    x = _c(x)
+    C, H, W = x.shape
+    y = np.empty_like(x)
+    load().oracle_normalize(_p(x), _p(y), W, H, C, int(kind), ctypes.c_float(target_mean), ctypes.c_float(target_dev))
+    return y
+
+
+def normalize_f64(x, kind, target_mean=0.0, target_dev=1.0):
+    """Closed form in float64: population mean / standard deviation over the whole tensor."""
+    x64 = np.asarray(x, np.float64)
+    add = target_mean - x64.mean() if kind != 1 else 0.0
+    mul = target_dev / x64.std() if kind != 0 else 1.0
+    return (x64 + add) * mul
+
+
 def slice3d(x, origin, shape):
     """origin (x,y,z), shape (w,h,c) on x [C,H,W]."""
     x = _c(x)
@@ -268,6 +285,9 @@ def run_spec(spec, feeds, force_direct=False, f64=False):
             v = slice3d(outs[n["in"]], n["origin"], n["shape"])
         elif op == "scalar":
             v = scalar_op(outs[n["in"]], n["kind"], n["value"])
+        elif op == "norm":
+            v = normalize_f64(outs[n["in"]], n["kind"], n["mean"], n["dev"]).astype(np.float32) if f64 else \
+                normalize(outs[n["in"]], n["kind"], n["mean"], n["dev"])
         else:
             raise ValueError("unknown op %r" % op)
         outs.append(v)
@@ -311,6 +331,8 @@ def parse_graph_dir(path):
             node = {"op": "concat", "ins": prev, "dim": int(params[1])}
         elif desc.startswith("ElemWise1Op"):
             node = {"op": "scalar", "in": prev[0], "kind": int(params[0]), "value": float(params[1])}
+        elif desc.startswith("Normalization"):
+            node = {"op": "norm", "in": prev[0], "kind": int(params[0]), "mean": float(params[1]), "dev": float(params[2])}
         else:
             raise ValueError("node type %s not part of the CNN layer path" % desc)
         spec[nid] = node

@@ -168,6 +168,21 @@ def test_fc_chain_fused(oracle, gpu):
     assert rel_err(res["1"], want[3]) <= LAYER_TOL and int(res["1"].argmax()) == int(want[3].argmax())
 
 
+def test_squeezenet_with_normalization_node(oracle, gpu):
+    """Config 4 with its per-image normalisation moved into the graph: raw U[0,255) image in, a
+    Normalization node (mean 0, deviation 1) in front of conv1."""
+    spec, feeds, got = run_config("squeezenet", size=96, normalise_in_graph=True)
+    assert spec[1]["op"] == "norm" and float(feeds[0].max()) > 100.0
+    want = oracle.run_spec(spec, feeds)
+    for i in got:
+        assert rel_err(got[i], want[i]) <= LAYER_TOL
+    assert int(got[len(spec) - 1].argmax()) == int(want[-1].argmax())
+    # the node alone, as an output
+    _, _, only = run_config("squeezenet", outputs=[1], size=96, normalise_in_graph=True)
+    assert rel_err(only[1], want[1]) <= LAYER_TOL
+    assert abs(float(only[1].astype(np.float64).mean())) < 1e-4 and abs(float(only[1].astype(np.float64).std()) - 1.0) < 1e-4
+
+
 def test_config4_squeezenet(oracle, gpu):
     spec, feeds, got = run_config("squeezenet", outputs=all_compute_nodes)
     want = check_layers(oracle, spec, feeds, got)

@@ -285,6 +285,25 @@ def test_fc_chain_without_finishing_kernels(lib, dev, oracle):
     assert lib.drhip_fc_ex_f32(xd, None, W1d, b1d, None, None, 64, 8, 0, 1, None) == -1        # unsplit layers cannot defer
 
 
+@pytest.mark.parametrize("C,H,W", [(3, 224, 224), (1, 5, 7), (4, 17, 33), (64, 56, 56), (1, 1, 2)])
+def test_normalize(lib, dev, oracle, C, H, W):
+    x = (np.random.default_rng(C + H).random((C, H, W), dtype=np.float32) * 255.0).astype(np.float32)
+    n = x.size
+    scratch = dev.empty(lib.drhip_normalize_scratch_floats(n))
+    xd, y = dev.put(x), dev.empty(n)
+    for kind, tm, td in [(0, 3.0, 1.0), (1, 0.0, 2.0), (2, 0.0, 1.0), (2, 0.5, 1.5)]:
+        first = None
+        for _ in range(2):                   # the scratch needs no reset between calls; fixed summation order
+            ok(lib, lib.drhip_normalize_f32(xd, y, n, kind, tm, td, scratch, None))
+            got = dev.get(y, x.shape)
+            assert first is None or np.array_equal(first, got)
+            first = got
+        assert rel_err(got, oracle.normalize(x, kind, tm, td)) <= TOL
+        assert rel_err(got, oracle.normalize_f64(x, kind, tm, td)) <= TOL
+    assert lib.drhip_normalize_f32(xd, y, n, 3, 0.0, 1.0, scratch, None) == -1
+    assert lib.drhip_normalize_f32(xd, y, 0, 2, 0.0, 1.0, scratch, None) == -1
+
+
 def test_softmax(lib, dev, oracle):
     for n, scale in [(1000, 3.0), (10, 1.0), (5000, 5.0), (1, 1.0)]:
         x = rnd(n, scale=scale)

@@ -136,6 +136,35 @@ def test_loader_error_paths(lib, tmp_path):
             dr.load_graph(g, MODEL)
 
 
+def test_normalization_node_format_roundtrip(lib, tmp_path):
+    """graph.dr grammar of the Normalization node: 3 parameters `type mean dev` written with %d %f %f
+    (reference src/dR_nodes_misc.c:1103-1105), read back into the same node."""
+    with dr.Environment() as env:
+        g = env.create_graph()
+        f = dr.feed_node(g, [6, 5, 3])
+        n = dr.Normalization(f, "target_mean_dev", 0.25, 2.0)
+        dr.Softmax(n)
+        dr.save_graph(g, str(tmp_path))
+    lines = open(tmp_path / "dr_graph_export" / "graph.dr").read().split("\n")
+    assert lines[6:11] == ["Node 1: Normalization", "params: 2 0.250000 2.000000", "previous_nodes: 0", "next_nodes: 2", "variable_files:"]
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes, feeds = dr.load_graph(g, str(tmp_path / "dr_graph_export"))
+        assert [dr.node_struct(x).type for x in nodes] == [12, 7, 14]          # feed, normalization, softmax
+        assert lib.dR_propagateShapesAndSchedule(g.ptr) == 1
+        s = dr.node_struct(nodes[1]).oshape
+        f0 = dr.node_struct(nodes[0]).oshape
+        assert (s.s0, s.s1, s.s2) == (f0.s0, f0.s1, f0.s2) and sorted((s.s0, s.s1, s.s2)) == [3, 5, 6]
+        dr.save_graph(g, str(tmp_path / "again"))
+    assert filecmp.cmp(str(tmp_path / "again" / "dr_graph_export" / "graph.dr"), str(tmp_path / "dr_graph_export" / "graph.dr"), shallow=False)
+    # wrong parameter count / unknown type are refused
+    feed = "Node 0: DataFeedNode\nparams: 4 4 2\nprevious_nodes:\nnext_nodes: 1\nvariable_files:\n"
+    _expect_load_failure(tmp_path, "deepRACIN graph: 2 nodes, 1 feed nodes\n" + feed +
+                         "Node 1: Normalization\nparams: 2 0.0\nprevious_nodes: 0\nnext_nodes:\nvariable_files:\n")
+    _expect_load_failure(tmp_path, "deepRACIN graph: 2 nodes, 1 feed nodes\n" + feed +
+                         "Node 1: Normalization\nparams: 5 0.0 1.0\nprevious_nodes: 0\nnext_nodes:\nvariable_files:\n")
+
+
 # ---------------------------------------------------------------------------------------------
 # prepare-time errors (host side only: fail before any device call)
 # ---------------------------------------------------------------------------------------------

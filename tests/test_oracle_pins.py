@@ -218,6 +218,33 @@ def test_softmax_matches_scipy(oracle):
     assert int(got.argmax()) == int(x.argmax())
 
 
+@pytest.mark.parametrize("C,H,W", [(3, 224, 224), (1, 5, 7), (4, 17, 33), (2, 8, 16), (5, 1, 1)])
+def test_normalize_matches_numpy_mean_and_std(oracle, C, H, W):
+    """Normalization node: mean and POPULATION standard deviation over the whole tensor (numpy's
+    float64 mean / std are the library routines the closed form reduces to), deviation about the mean
+    for type 1 too.  A sample deviation (n-1), a per-channel statistic or a dropped mean would fail."""
+    rng = np.random.default_rng(C * 100 + H)
+    x = (rng.random((C, H, W), dtype=np.float32) * 255.0 + np.arange(C, dtype=np.float32)[:, None, None] * 40.0).astype(np.float32)
+    x64 = x.astype(np.float64)
+    n = x.size
+    y0 = oracle.normalize(x, 0, 3.0, 1.0)
+    assert abs(float(y0.astype(np.float64).mean()) - 3.0) < 1e-3 and np.allclose(y0, x64 + (3.0 - x64.mean()), rtol=1e-5, atol=1e-3)
+    if n > 1:
+        y1 = oracle.normalize(x, 1, 0.0, 2.0)
+        assert np.allclose(y1, x64 * (2.0 / x64.std()), rtol=1e-4, atol=1e-4)
+        assert abs(float(y1.astype(np.float64).std()) - 2.0) < 1e-3
+        y2 = oracle.normalize(x, 2, 0.5, 1.5)
+        # (x + (0.5 - mean)) * (1.5 / std), Kernels/dR_math.cl:143: the target mean is scaled as well
+        want = (x64 - x64.mean()) / x64.std() * 1.5 + 0.5 * 1.5 / x64.std()
+        assert np.allclose(y2, want, rtol=1e-4, atol=1e-4)
+        assert np.allclose(y2, oracle.normalize_f64(x, 2, 0.5, 1.5), rtol=1e-4, atol=1e-4)
+        assert abs(float(y2.astype(np.float64).std()) - 1.5) < 1e-3
+        if C > 1:     # one statistic for the whole tensor, not one per channel
+            assert abs(float(y2[0].astype(np.float64).mean()) - float(y2[-1].astype(np.float64).mean())) > 0.1
+    # invariances that fix signs: shifting the input does not change a mean-normalised output
+    assert np.allclose(oracle.normalize(x + np.float32(10.0), 0, 0.0, 1.0), oracle.normalize(x, 0, 0.0, 1.0), atol=2e-3)
+
+
 def test_scalar_concat_slice(oracle):
     x = rnd(4, 3, 5)
     assert np.array_equal(oracle.scalar_op(x, 1, 2.5), x - np.float32(2.5))
