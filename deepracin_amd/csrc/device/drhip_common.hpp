@@ -65,6 +65,25 @@ inline void launch(Kernel kernel, dim3 grid, dim3 block, size_t ldsBytes, hipStr
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Element `row` of an activation vector that a split GEMV left as partial sums: slices added in
+// order, then bias and ReLU -- bit for bit what the GEMV's finishing kernel stores.
+__device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {
+    const float* pp = d.partials + row;
+    float s = 0.0f;
+    int sl = 0;
+    for (; sl + 8 <= d.slices; sl += 8) {           // 8 independent loads in flight, summed in slice order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = pp[(size_t)(sl + u) * d.n];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s += v[u];
+    }
+    for (; sl < d.slices; ++sl) s += pp[(size_t)sl * d.n];
+    if (d.bias) s += d.bias[row];
+    if (d.relu) s = fmaxf(s, 0.0f);
+    return s;
+}
+
 // Number of compute units of the active device (cached by drhip_init; 256 on MI355X).
 int num_cu();
 

@@ -64,24 +64,6 @@ static FcPlan fc_plan(int K, int N) {
 
 // Partial GEMV of one (column panel, row slice).  slices == 1: writes y directly (bias, ReLU).
 // Otherwise writes partials[slice][n]; fc_reduce_kernel finishes.
-// Element `row` of an activation vector left as partial sums: slices added in order, then bias, ReLU.
-__device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {
-    const float* pp = d.partials + row;
-    float s = 0.0f;
-    int sl = 0;
-    for (; sl + 8 <= d.slices; sl += 8) {           // 8 independent loads in flight, summed in slice order
-        float v[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = pp[(size_t)(sl + u) * d.n];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) s += v[u];
-    }
-    for (; sl < d.slices; ++sl) s += pp[(size_t)sl * d.n];
-    if (d.bias) s += d.bias[row];
-    if (d.relu) s = fmaxf(s, 0.0f);
-    return s;
-}
-
 template <int VEC, bool DEFERRED>
 __global__ void __launch_bounds__(kFcThreads)
 fc_gemv_kernel(const float* __restrict__ x, drhip_deferred_vec xdef, const float* __restrict__ Wt,
@@ -107,6 +89,7 @@ fc_gemv_kernel(const float* __restrict__ x, drhip_deferred_vec xdef, const float
         const int rows = min(kWave, rowEnd - r0);
         const float xraw = DEFERRED ? deferred_element(xdef, min(r0 + lane, K - 1)) : x[min(r0 + lane, K - 1)];
         const float xl = (lane < rows) ? xraw : 0.0f;
+        if (DEFERRED && xdef.finished && panel == 0 && lane < rows) xdef.finished[r0 + lane] = xraw;   // each row once
         const float* wp = Wt + (size_t)r0 * N + col;
         if (rows == kWave) {
             // 64 rows as 8 batches of 8 row loads; two batches (16 KiB per wave) are always in flight
@@ -225,7 +208,7 @@ extern "C" int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, c
     DRHIP_REQUIRE(p.slices <= 65535, "drhip_fc_f32: too many row slices");
     dim3 grid(p.panels, p.slices);
     hipStream_t s = as_stream(stream);
-    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0};
+    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0, nullptr};
     const drhip_deferred_vec& xd = xdef ? *xdef : none;
     if (p.vec == 4) launch_gemv<4>(xdef != nullptr, grid, s, x, xd, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu, defer);
     else if (p.vec == 2) launch_gemv<2>(xdef != nullptr, grid, s, x, xd, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu, defer);

@@ -23,7 +23,8 @@ __device__ inline float wave_sum(float v) {
 }
 
 // xdef.partials != NULL: the logits arrive as the partial sums of the GEMV in front (slices added
-// in order, then its bias and ReLU); they are finished into y first, which then serves as x.
+// in order, then its bias and ReLU); they are finished into y first (and into xdef.finished, when
+// the caller wants to read the logits too), which then serves as x.
 __global__ void __launch_bounds__(kSoftmaxThreads)
 softmax_kernel(const float* x, drhip_deferred_vec xdef, float* y, int n) {     // no __restrict__: x may become y
     __shared__ float red[kSoftmaxThreads / kWave];
@@ -32,12 +33,9 @@ softmax_kernel(const float* x, drhip_deferred_vec xdef, float* y, int n) {     /
     constexpr int nwaves = kSoftmaxThreads / kWave;
     if (xdef.partials) {
         for (int i = tid; i < n; i += kSoftmaxThreads) {
-            const float* pp = xdef.partials + i;
-            float s = 0.0f;
-            for (int sl = 0; sl < xdef.slices; ++sl) s += pp[(size_t)sl * xdef.n];
-            if (xdef.bias) s += xdef.bias[i];
-            if (xdef.relu) s = fmaxf(s, 0.0f);
+            const float s = deferred_element(xdef, i);
             y[i] = s;                           // every lane re-reads only the elements it wrote itself
+            if (xdef.finished) xdef.finished[i] = s;
         }
         x = y;
     }
@@ -79,7 +77,8 @@ extern "C" int drhip_softmax_ex_f32(const float* x, const drhip_deferred_vec* xd
     DRHIP_REQUIRE((x || xdef) && y, "drhip_softmax_f32: NULL tensor");
     DRHIP_REQUIRE(n > 0, "drhip_softmax_f32: n = %d", n);
     DRHIP_REQUIRE(!xdef || (xdef->partials && xdef->slices > 0 && xdef->n == n), "drhip_softmax_f32: deferred input must carry partial sums of a vector of length %d", n);
-    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0};
+    DRHIP_REQUIRE(!xdef || xdef->finished != y, "drhip_softmax_f32: the finished logits and the probabilities need separate arrays");
+    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0, nullptr};
     launch(softmax_kernel, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, xdef ? *xdef : none, y, n);
     return launched("softmax_kernel");
 }

@@ -167,6 +167,10 @@ gboolean dR_prepare(dR_Graph* net) {
     const bool talk = verbose(net);
     if (!ensure_device(net)) { say("dR_initCL Failed \n"); return FALSE; }
 
+    // a second dR_prepare plans new buffers: the recorded launch graph of the old ones must go
+    if (net->drGraphExec) { drhip_graph_destroy(net->drGraphExec); net->drGraphExec = NULL; }
+    net->drGraphOff = FALSE;
+
     if (talk) say("Propagate shapes and schedule...\n");
     if (!dR_propagateShapesAndSchedule(net)) { say("dR_propagateShapesAndSchedule Failed \n"); return FALSE; }
     if (talk) say("Done.\n");
@@ -205,6 +209,10 @@ gint dR_getOutputBuffers(dR_Graph* net, cl_mem** outptr) {
 }
 
 void dR_feedData(dR_Graph* net, dR_Node* feednode, gfloat* data, gint offset, gint numfloats) {
+    if (!feednode || !feednode->outputBuf || offset < 0 || numfloats < 0) {
+        say("dR_feedData: feed node has no buffer yet (call dR_prepare first) or bad range\n");
+        return;
+    }
     dR_uploadArray(net, (gchar*)"", data, (size_t)offset * sizeof(float), (size_t)numfloats * sizeof(float),
                    feednode->outputBuf->buf);
 }
@@ -216,11 +224,10 @@ void dR_feedData(dR_Graph* net, dR_Node* feednode, gfloat* data, gint offset, gi
 // be captured (it blocks or allocates) keep the node-by-node path.
 //
 // profilingGPU: the reference waits for every kernel and reads its cl_event (src/dR_clwrap.c:970-1049).
-// Here one hipEvent is recorded between consecutive nodes while the whole pass is enqueued without
-// waiting; after the last node the pass is awaited once and the differences of neighbouring events
-// give each node's device time (node->drLastKernelMs) and their sum (clConfig->totalKernelGPUTime,
-// printed like the reference does).  The stream therefore runs at its natural pace and the times
-// are not inflated by host launch latency.
+// Here every kernel launch of the pass carries its own start/stop events while the pass is enqueued
+// without waiting; after the last node the pass is awaited once, a node's device time
+// (node->drLastKernelMs) is the sum over its kernels, and their sum goes to
+// clConfig->totalKernelGPUTime, printed like the reference does.
 gboolean dR_apply(dR_Graph* net) {
     if (!net->prepared) { say("dR_apply: graph is not prepared. Call dR_prepare first! \n"); return FALSE; }
     dR_ClConfig* cc = net->clConfig;

@@ -154,6 +154,7 @@ drhip_deferred_vec deferred_output_of(dR_Node* producer) {
     d.slices = drhip_fc_slices(p->shape.s0, p->shape.s1);
     d.n = p->shape.s1;
     d.relu = p->activation == tReLU;
+    d.finished = producer->output ? dev_out(producer) : NULL;   // the caller reads this tensor as well
     return d;
 }
 

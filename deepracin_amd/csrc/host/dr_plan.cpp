@@ -209,7 +209,8 @@ gboolean dR_planBuffers(dR_Graph* net) {
     for (dR_Node* n : sched) {
         if (n->type != tFullyConnected || (fuseFc && strcmp(fuseFc, "0") == 0)) continue;
         dR_FC_Data* fd = (dR_FC_Data*)n->layer;
-        if (n->output || n->outputBuf || !n->next_layers || n->next_layers->length != 1) continue;
+        // an output node can defer too: its consumer stores the finished vector into its buffer
+        if (n->outputBuf || !n->next_layers || n->next_layers->length != 1) continue;
         if (drhip_fc_slices(fd->shape.s0, fd->shape.s1) <= 1) continue;
         dR_Node* c = nodes_of(n->next_layers)[0];
         if (c->type == tFullyConnected) ((dR_FC_Data*)c->layer)->drDeferredInput = n;

@@ -169,12 +169,15 @@ int drhip_fc_f32(const float* x, const float* Wt, const float* bias, float* y,
  * the consumer is told where the sums are through a drhip_deferred_vec: element k of that vector is
  * act(bias[k] + sum_{s < slices} partials[s*n + k]), slices added in order - the value, bit for bit,
  * that the finishing kernel would have stored.  drhip_fc_ex_f32 and drhip_softmax_ex_f32 accept
- * such a vector as their input (`xdef` != NULL; x is then ignored).  No counterpart in the
+ * such a vector as their input (`xdef` != NULL; x is then ignored) and, when `finished` is set,
+ * store it there on the way.  No counterpart in the
  * reference, which always runs its second kernel (src/dR_nodes_fc.c:239-275). */
 typedef struct drhip_deferred_vec {
     const float* partials;   /* [slices][n] */
     const float* bias;       /* [n] or NULL */
     int slices, n, relu;
+    float* finished;         /* NULL, or [n]: the consumer also stores the finished vector here (for a
+                                producer whose own output the caller wants to read) */
 } drhip_deferred_vec;
 int drhip_fc_slices(int K, int N);
 int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, const float* Wt, const float* bias, float* y,

@@ -166,6 +166,20 @@ def test_fc_chain_fused(oracle, gpu):
     assert np.array_equal(res["1"], res["0"])
     want = oracle.run_spec(spec, {0: x})
     assert rel_err(res["1"], want[3]) <= LAYER_TOL and int(res["1"].argmax()) == int(want[3].argmax())
+    # Both GEMV outputs wanted by the caller as well: still 3 launches, the consumers store the
+    # finished vectors into the producers' output buffers on the way.
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes = configs.build_graph(g, spec, [1, 2, 3])
+        dr.prepare(g)
+        configs.feed_chw(nodes[0], x)
+        assert g.lib.dR_apply(g.ptr) and g.lib.dR_apply(g.ptr)
+        outs = [a.copy() for a in configs.fetch_chw(g)]
+        dr.graph_config(g).profilingGPU = 1
+        assert g.lib.dR_apply(g.ptr) and g.lib.drhip_timing_count() == 3
+    assert np.array_equal(outs[2], res["0"])
+    for k in range(3):
+        assert rel_err(outs[k], want[k + 1]) <= LAYER_TOL
 
 
 def test_squeezenet_with_normalization_node(oracle, gpu):

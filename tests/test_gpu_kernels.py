@@ -248,7 +248,7 @@ def test_fc(lib, dev, oracle, C, H, W, N, relu):
 
 class DeferredVec(ctypes.Structure):
     """drhip_deferred_vec (include/dr_hip.h)."""
-    _fields_ = [("partials", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("slices", ctypes.c_int), ("n", ctypes.c_int), ("relu", ctypes.c_int)]
+    _fields_ = [("partials", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("slices", ctypes.c_int), ("n", ctypes.c_int), ("relu", ctypes.c_int), ("finished", ctypes.c_void_p)]
 
 
 def test_fc_chain_without_finishing_kernels(lib, dev, oracle):
@@ -266,21 +266,31 @@ def test_fc_chain_without_finishing_kernels(lib, dev, oracle):
     ok(lib, lib.drhip_fc_f32(xd, W1d, b1d, y1, p1, K, N1, 1, None))
     ok(lib, lib.drhip_fc_f32(y1, W2d, b2d, y2, p2, N1, N2, 0, None))
     ok(lib, lib.drhip_softmax_f32(y2, prob, N2, None))
-    want2, wantp = dev.get(y2, (N2,)), dev.get(prob, (N2,))
+    want1, want2, wantp = dev.get(y1, (N1,)), dev.get(y2, (N2,)), dev.get(prob, (N2,))
     assert rel_err(want2, oracle.fc(oracle.fc(x.reshape(K, 1, 1), W1, b1, relu=True), W2, b2, relu=False).reshape(-1)) <= TOL
     # deferred chain: y1 and y2 are never written
     q1, q2, prob2 = dev.empty(s1 * N1), dev.empty(s2 * N2), dev.empty(N2)
     ok(lib, lib.drhip_fc_ex_f32(xd, None, W1d, b1d, None, q1, K, N1, 1, 1, None))
-    d1 = DeferredVec(q1.value, b1d.value, s1, N1, 1)
+    d1 = DeferredVec(q1.value, b1d.value, s1, N1, 1, None)
     y2b = dev.empty(N2)
     ok(lib, lib.drhip_fc_ex_f32(None, ctypes.byref(d1), W2d, b2d, y2b, q2, N1, N2, 0, 0, None))
     assert np.array_equal(dev.get(y2b, (N2,)), want2)
     ok(lib, lib.drhip_fc_ex_f32(None, ctypes.byref(d1), W2d, b2d, None, q2, N1, N2, 0, 1, None))
-    d2 = DeferredVec(q2.value, b2d.value, s2, N2, 0)
+    d2 = DeferredVec(q2.value, b2d.value, s2, N2, 0, None)
     ok(lib, lib.drhip_softmax_ex_f32(None, ctypes.byref(d2), prob2, N2, None))
     assert np.array_equal(dev.get(prob2, (N2,)), wantp)
+    # ... and with the consumers also storing the finished vectors (producers whose output is wanted too)
+    fin1, fin2 = dev.put(np.full(N1, -7.0, np.float32)), dev.put(np.full(N2, -7.0, np.float32))
+    d1f = DeferredVec(q1.value, b1d.value, s1, N1, 1, fin1.value)
+    ok(lib, lib.drhip_fc_ex_f32(None, ctypes.byref(d1f), W2d, b2d, None, q2, N1, N2, 0, 1, None))
+    assert np.array_equal(dev.get(fin1, (N1,)), want1)
+    d2f = DeferredVec(q2.value, b2d.value, s2, N2, 0, fin2.value)
+    ok(lib, lib.drhip_softmax_ex_f32(None, ctypes.byref(d2f), prob2, N2, None))
+    assert np.array_equal(dev.get(prob2, (N2,)), wantp) and np.array_equal(dev.get(fin2, (N2,)), want2)
+    d2bad = DeferredVec(q2.value, b2d.value, s2, N2, 0, prob2.value)
+    assert lib.drhip_softmax_ex_f32(None, ctypes.byref(d2bad), prob2, N2, None) == -1
     # argument checks
-    bad = DeferredVec(q1.value, b1d.value, s1, N1 + 1, 1)
+    bad = DeferredVec(q1.value, b1d.value, s1, N1 + 1, 1, None)
     assert lib.drhip_fc_ex_f32(None, ctypes.byref(bad), W2d, b2d, y2b, q2, N1, N2, 0, 0, None) == -1
     assert lib.drhip_fc_ex_f32(xd, None, W1d, b1d, None, None, 64, 8, 0, 1, None) == -1        # unsplit layers cannot defer
 
