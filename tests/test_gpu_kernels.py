@@ -340,3 +340,85 @@ def test_copy3d_and_scalar(lib, dev, oracle):
         y = dev.empty(x.size)
         ok(lib, lib.drhip_scalar_op_f32(dev.put(x), y, x.size, op, s, None))
         assert np.array_equal(dev.get(y, x.shape), oracle.scalar_op(x, op, s))
+
+
+# ---------------------------------------------------------------------------------------------
+# Seeded sweeps over ragged shapes: sizes that are no multiple of any tile, panel, stage or vector
+# width the kernels use, single rows / columns / channels included.
+
+def _sweep(seed, count, draw):
+    rng = np.random.default_rng(seed)
+    return [draw(rng) for _ in range(count)]
+
+
+@pytest.mark.parametrize("W,H,I,O,variant", _sweep(11, 24, lambda r: (
+    int(r.integers(1, 41)), int(r.integers(1, 41)), int(r.integers(1, 41)), int(r.integers(1, 71)),
+    int(r.choice([0, 1, 2, 3, 0x11, 0x12, 0x21, 0x31]))))
+    + [(1, 37, 9, 31, 0x11), (37, 1, 8, 32, 1), (3, 3, 64, 33, 0x21), (40, 2, 17, 1, 2)])
+def test_winograd_sweep(lib, dev, oracle, W, H, I, O, variant):
+    x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
+    U, _ = wino_filters(lib, dev, w)
+    ws = wino_workspace(lib, dev, W, H, I, O, variant)
+    relu = (W + H + I + O) & 1
+    want = oracle.conv_winograd(x, w, b, relu=bool(relu))
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, H, I, O, relu, variant, ws, None))
+    got = dev.get(out, want.shape)
+    assert rel_err(got, want) <= TOL and rel_err(got, oracle.conv_f64(x, w, b, relu=bool(relu))) <= TOL
+
+
+@pytest.mark.parametrize("W,H,I,O,kw,kh,sx,sy", _sweep(12, 20, lambda r: (
+    int(r.integers(1, 40)), int(r.integers(1, 40)), int(r.integers(1, 20)), int(r.integers(1, 40)),
+    int(r.choice([1, 3, 5, 7])), int(r.choice([1, 3, 5])), int(r.integers(1, 4)), int(r.integers(1, 4)))))
+def test_conv_direct_sweep(lib, dev, oracle, W, H, I, O, kw, kh, sx, sy):
+    if W // sx == 0 or H // sy == 0:
+        pytest.skip("empty output")
+    x, w, b = rnd(I, H, W), rnd(I, O, kh, kw, scale=np.sqrt(2.0 / (kh * kw * I))), rnd(O, scale=0.01)
+    want = oracle.conv_direct(x, w, b, (sx, sy), relu=False)
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_conv2d_direct_f32(dev.put(x), dev.put(w), dev.put(b), out, W, H, I, O, kw, kh, sx, sy, 0, None))
+    got = dev.get(out, want.shape)
+    assert rel_err(got, want) <= TOL and rel_err(got, oracle.conv_f64(x, w, b, stride=(sx, sy))) <= TOL
+
+
+@pytest.mark.parametrize("P,I,O,variant", _sweep(13, 20, lambda r: (
+    int(r.integers(1, 400)), int(r.integers(1, 100)), int(r.integers(1, 100)), int(r.choice([0, 1, 2, 4, 8])))))
+def test_conv1x1_sweep(lib, dev, oracle, P, I, O, variant):
+    x, w, b = rnd(I, 1, P), rnd(I, O, 1, 1, scale=np.sqrt(2.0 / I)), rnd(O, scale=0.01)
+    want = oracle.conv1x1(x, w, b, relu=False)
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_conv1x1_f32(dev.put(x), dev.put(w), dev.put(b), out, P, I, O, 0, variant, None))
+    assert rel_err(dev.get(out, want.shape), want) <= TOL
+
+
+@pytest.mark.parametrize("W,H,C,kx,ky,kz,sx,sy,sz", _sweep(14, 24, lambda r: (
+    int(r.integers(1, 30)), int(r.integers(1, 30)), int(r.integers(1, 9)),
+    int(r.integers(1, 12)), int(r.integers(1, 12)), int(r.integers(1, 3)),
+    int(r.integers(1, 6)), int(r.integers(1, 6)), int(r.integers(1, 3)))))
+def test_pool_sweep(lib, dev, oracle, W, H, C, kx, ky, kz, sx, sy, sz):
+    x = rnd(C, H, W)
+    x[:, ::2, ::3] = x.flat[0]
+    for kind in (0, 1):
+        want = oracle.pool(x, (kx, ky, kz), (sx, sy, sz), kind)
+        out = dev.empty(want.size)
+        ok(lib, lib.drhip_pool_f32(dev.put(x), out, None, W, H, C, kx, ky, kz, sx, sy, sz, kind, None))
+        got = dev.get(out, want.shape)
+        if kind == 0:
+            assert np.array_equal(got, want)
+        else:
+            assert rel_err(got, want) <= 1e-6
+
+
+@pytest.mark.parametrize("C,H,W,N", _sweep(15, 16, lambda r: (
+    int(r.integers(1, 70)), int(r.integers(1, 6)), int(r.integers(1, 6)), int(r.integers(1, 600)))))
+def test_fc_sweep(lib, dev, oracle, C, H, W, N):
+    K = C * H * W
+    x, Wt, b = rnd(C, H, W), rnd(K, N, scale=np.sqrt(2.0 / K)), rnd(N, scale=0.01)
+    want = oracle.fc(x, Wt, b, relu=False).reshape(-1)
+    perm = dev.empty(K * N)
+    ok(lib, lib.drhip_fc_permute_rows_f32(dev.put(Wt), perm, W, H, C, N, None))
+    n = lib.drhip_fc_scratch_floats(K, N)
+    y = dev.empty(N)
+    ok(lib, lib.drhip_fc_f32(dev.put(x), perm, dev.put(b), y, dev.empty(n) if n else None, K, N, 0, None))
+    got = dev.get(y, (N,))
+    assert rel_err(got, want) <= TOL and rel_err(got, oracle.fc_f64(x, Wt, b).reshape(-1)) <= TOL
