@@ -334,3 +334,89 @@ def test_launch_graph_replays_equal_node_by_node(gpu, name):
         for x, y in zip(a, b):
             assert np.array_equal(x, y), "replay %d differs from the node-by-node pass" % k
     assert np.array_equal(replay[0][0], replay[-1][0])
+
+
+# ---------------------------------------------------------------------------------------------
+# Random topologies: the buffer planner (live intervals, fused concats, pooled convolutions, joint
+# expand launches, deferred GEMV reductions) must give the oracle's values whatever the graph looks
+# like and whichever subset of nodes the caller reads.
+
+def _random_spec(seed):
+    rng = np.random.default_rng(seed)
+    W, H, C = int(rng.integers(5, 30)), int(rng.integers(5, 30)), int(rng.integers(1, 9))
+    spec = [{"op": "feed", "shape": (W, H, C)}]
+    shapes = [(W, H, C)]
+
+    def conv(src, k, cout, stride=1, relu=True):
+        cin = shapes[src][2]
+        w = (rng.standard_normal((cin, cout, k, k)) * np.sqrt(2.0 / (k * k * cin))).astype(np.float32)
+        b = (rng.standard_normal(cout) * 0.05).astype(np.float32) if rng.random() < 0.8 else None
+        spec.append({"op": "conv", "in": src, "w": w, "b": b, "stride": (stride, stride), "relu": relu})
+        shapes.append((shapes[src][0] // stride, shapes[src][1] // stride, cout))
+        return len(spec) - 1
+
+    cur = 0
+    for _ in range(int(rng.integers(3, 8))):
+        w_, h_, c_ = shapes[cur]
+        kind = rng.choice(["conv3", "conv1", "conv5", "pool2", "pool3", "fire", "branch3", "slice", "scalar", "norm"])
+        if kind == "conv3":
+            cur = conv(cur, 3, int(rng.integers(1, 40)), relu=bool(rng.integers(0, 2)))
+        elif kind == "conv1":
+            cur = conv(cur, 1, int(rng.integers(1, 40)))
+        elif kind == "conv5" and min(w_, h_) >= 4:
+            cur = conv(cur, 5, int(rng.integers(1, 12)), stride=int(rng.integers(1, 3)))
+        elif kind in ("pool2", "pool3") and min(w_, h_) >= 2:
+            k, s = (2, 2) if kind == "pool2" else (3, 2)
+            spec.append({"op": "pool", "in": cur, "window": (k, k, 1), "stride": (s, s, 1), "kind": int(rng.integers(0, 2))})
+            shapes.append((-(-w_ // s), -(-h_ // s), c_)); cur = len(spec) - 1
+        elif kind == "fire":
+            s = conv(cur, 1, int(rng.integers(1, 12)))
+            e = int(rng.integers(1, 40))
+            a, b = conv(s, 1, e), conv(s, 3, e)
+            spec.append({"op": "concat", "ins": [a, b], "dim": 2}); shapes.append((w_, h_, 2 * e)); cur = len(spec) - 1
+        elif kind == "branch3":                      # three producers, one of them read twice
+            a, b = conv(cur, 3, int(rng.integers(1, 10))), conv(cur, 1, int(rng.integers(1, 10)))
+            ins = [a, b, cur] if rng.random() < 0.5 else [b, a, a]
+            spec.append({"op": "concat", "ins": ins, "dim": 2})
+            shapes.append((w_, h_, sum(shapes[i][2] for i in ins))); cur = len(spec) - 1
+        elif kind == "slice" and c_ >= 2:
+            z0 = int(rng.integers(0, c_ - 1)); cz = int(rng.integers(1, c_ - z0 + 1))
+            x0 = int(rng.integers(0, w_)); cw = int(rng.integers(1, w_ - x0 + 1))
+            spec.append({"op": "slice", "in": cur, "origin": (x0, 0, z0), "shape": (cw, h_, cz)})
+            shapes.append((cw, h_, cz)); cur = len(spec) - 1
+        elif kind == "scalar":
+            spec.append({"op": "scalar", "in": cur, "kind": int(rng.integers(0, 3)), "value": float(rng.uniform(0.5, 2.0))})
+            shapes.append(shapes[cur]); cur = len(spec) - 1
+        elif kind == "norm" and w_ * h_ * c_ > 1:
+            spec.append({"op": "norm", "in": cur, "kind": int(rng.integers(0, 3)), "mean": 0.25, "dev": 1.5})
+            shapes.append(shapes[cur]); cur = len(spec) - 1
+    if rng.random() < 0.6:                           # classifier tail
+        w_, h_, c_ = shapes[cur]
+        for n_out, relu in ((int(rng.integers(200, 700)), True), (int(rng.integers(2, 300)), False)):
+            k = shapes[cur][0] * shapes[cur][1] * shapes[cur][2]
+            spec.append({"op": "fc", "in": cur, "w": (rng.standard_normal((k, n_out)) * np.sqrt(2.0 / k)).astype(np.float32),
+                         "b": (rng.standard_normal(n_out) * 0.05).astype(np.float32), "relu": relu})
+            shapes.append((n_out, 1, 1)); cur = len(spec) - 1
+        spec.append({"op": "softmax", "in": cur}); shapes.append(shapes[cur]); cur = len(spec) - 1
+    x = rng.random((C, H, W), dtype=np.float32) + np.float32(0.1)
+    compute = [i for i in range(1, len(spec))]
+    some = sorted(set([cur] + [int(i) for i in rng.choice(compute, size=min(2, len(compute)), replace=False)]))
+    return spec, x, some
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_random_topologies(oracle, gpu, seed):
+    spec, x, some = _random_spec(1000 + seed)
+    want = oracle.run_spec(spec, {0: x})
+    for outs in (some, [i for i in range(1, len(spec))]):
+        with dr.Environment() as env:
+            g = env.create_graph()
+            nodes = configs.build_graph(g, spec, outs)
+            dr.prepare(g)
+            configs.feed_chw(nodes[0], x)
+            for _ in range(2):                           # the captured pass, then a replay
+                assert g.lib.dR_apply(g.ptr)
+                got = configs.fetch_chw(g)
+                for i, a in zip(outs, got):
+                    assert a.shape == want[i].shape, (seed, i, spec[i]["op"], a.shape, want[i].shape)
+                    assert rel_err(a, want[i]) <= LAYER_TOL, (seed, i, spec[i]["op"], [s["op"] for s in spec])
