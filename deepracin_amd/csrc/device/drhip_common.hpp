@@ -71,7 +71,16 @@ __device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {
     const float* pp = d.partials + row;
     float s = 0.0f;
     int sl = 0;
-    for (; sl + 8 <= d.slices; sl += 8) {           // 8 independent loads in flight, summed in slice order
+    // 32, then 8 independent loads in flight, always summed in slice order: the partial sums come
+    // from other XCDs' workgroups, so every round of loads costs a trip to memory
+    for (; sl + 32 <= d.slices; sl += 32) {
+        float v[32];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) v[u] = pp[(size_t)(sl + u) * d.n];
+#pragma unroll
+        for (int u = 0; u < 32; ++u) s += v[u];
+    }
+    for (; sl + 8 <= d.slices; sl += 8) {
         float v[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) v[u] = pp[(size_t)(sl + u) * d.n];

@@ -64,7 +64,10 @@ static FcPlan fc_plan(int K, int N) {
 
 // Partial GEMV of one (column panel, row slice).  slices == 1: writes y directly (bias, ReLU).
 // Otherwise writes partials[slice][n]; fc_reduce_kernel finishes.
-template <int VEC, bool DEFERRED>
+// CH = rows per wavefront and turn (64, 32 or 16): a wavefront fetches CH activations, one per lane,
+// and streams the CH matrix rows against them.  Short slices use a small CH so that all four
+// wavefronts of the workgroup have rows to stream.
+template <int VEC, bool DEFERRED, int CH>
 __global__ void __launch_bounds__(kFcThreads)
 fc_gemv_kernel(const float* __restrict__ x, drhip_deferred_vec xdef, const float* __restrict__ Wt,
                const float* __restrict__ bias, float* __restrict__ y, float* __restrict__ partials,
@@ -85,26 +88,31 @@ fc_gemv_kernel(const float* __restrict__ x, drhip_deferred_vec xdef, const float
 #pragma unroll
     for (int v = 0; v < VEC; ++v) acc[v] = 0.0f;
 
-    for (int r0 = rowBegin + wave * kWave; r0 < rowEnd; r0 += kFcWaves * kWave) {
-        const int rows = min(kWave, rowEnd - r0);
-        const float xraw = DEFERRED ? deferred_element(xdef, min(r0 + lane, K - 1)) : x[min(r0 + lane, K - 1)];
-        const float xl = (lane < rows) ? xraw : 0.0f;
-        if (DEFERRED && xdef.finished && panel == 0 && lane < rows) xdef.finished[r0 + lane] = xraw;   // each row once
+    for (int r0 = rowBegin + wave * CH; r0 < rowEnd; r0 += kFcWaves * CH) {
+        const int rows = min(CH, rowEnd - r0);
         const float* wp = Wt + (size_t)r0 * N + col;
-        if (rows == kWave) {
-            // 64 rows as 8 batches of 8 row loads; two batches (16 KiB per wave) are always in flight
-            vec_t wa[kFcUnroll], wb[kFcUnroll];
+        // The matrix stream starts before the activation is fetched: a deferred input costs a few
+        // rounds of loads of its own, and the weights must not wait behind them.
+        vec_t wa[kFcUnroll], wb[kFcUnroll];
+        if (rows == CH) {
 #pragma unroll
             for (int u = 0; u < kFcUnroll; ++u) wa[u] = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)u * N));
+        }
+        float xraw = 0.0f;
+        if (CH == kWave || lane < CH) xraw = DEFERRED ? deferred_element(xdef, min(r0 + lane, K - 1)) : x[min(r0 + lane, K - 1)];
+        const float xl = (lane < rows) ? xraw : 0.0f;
+        if (DEFERRED && xdef.finished && panel == 0 && lane < rows) xdef.finished[r0 + lane] = xraw;   // each row once
+        if (rows == CH) {
+            // CH rows as batches of 8 row loads; two batches (16 KiB per wave) are always in flight
 #pragma unroll
-            for (int j0 = 0; j0 < kWave; j0 += 2 * kFcUnroll) {
+            for (int j0 = 0; j0 < CH; j0 += 2 * kFcUnroll) {
 #pragma unroll
                 for (int u = 0; u < kFcUnroll; ++u)
                     wb[u] = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)(j0 + kFcUnroll + u) * N));
 #pragma unroll
                 for (int u = 0; u < kFcUnroll; ++u)
                     fma_row<VEC>(acc, wa[u], __int_as_float(__builtin_amdgcn_readlane(__float_as_int(xl), j0 + u)));
-                if (j0 + 2 * kFcUnroll < kWave) {
+                if (j0 + 2 * kFcUnroll < CH) {
 #pragma unroll
                     for (int u = 0; u < kFcUnroll; ++u)
                         wa[u] = __builtin_nontemporal_load((const vec_t*)(wp + (size_t)(j0 + 2 * kFcUnroll + u) * N));
@@ -188,11 +196,20 @@ extern "C" int drhip_fc_slices(int K, int N) {
     return fc_plan(K, N).slices;
 }
 
+template <int VEC, int CH>
+static void launch_gemv_ch(bool deferred, dim3 grid, hipStream_t s, const float* x, const drhip_deferred_vec& xd, const float* Wt,
+                           const float* bias, float* y, float* partials, int K, int N, int rowsPerSlice, int relu, int defer) {
+    if (deferred) launch((fc_gemv_kernel<VEC, true, CH>), grid, dim3(kFcThreads), 0, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
+    else launch((fc_gemv_kernel<VEC, false, CH>), grid, dim3(kFcThreads), 0, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
+}
+
 template <int VEC>
 static void launch_gemv(bool deferred, dim3 grid, hipStream_t s, const float* x, const drhip_deferred_vec& xd, const float* Wt,
                         const float* bias, float* y, float* partials, int K, int N, int rowsPerSlice, int relu, int defer) {
-    if (deferred) launch((fc_gemv_kernel<VEC, true>), grid, dim3(kFcThreads), 0, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
-    else launch((fc_gemv_kernel<VEC, false>), grid, dim3(kFcThreads), 0, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
+    // rows per wavefront and turn: every wavefront of the workgroup should get at least one turn
+    if (rowsPerSlice >= kFcWaves * kWave) launch_gemv_ch<VEC, 64>(deferred, grid, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
+    else if (rowsPerSlice >= kFcWaves * 32) launch_gemv_ch<VEC, 32>(deferred, grid, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
+    else launch_gemv_ch<VEC, 16>(deferred, grid, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
 }
 
 extern "C" int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, const float* Wt, const float* bias, float* y,

@@ -439,7 +439,8 @@ using namespace drhip;
 //   - 32 output channels per workgroup; 64 only for layers with very many tiles (224x224), where
 //     the panels alone give several workgroups per CU and sharing the input transform pays;
 //   - the input channels are split until at least ~160 workgroups exist, keeping at least 2 stages
-//     of 8 channels per split.
+//     of 8 channels per split;
+//   - split layers with very long channel loops trade panel width against split count.
 extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     const int T = ((W + 1) / 2) * ((H + 1) / 2);
     const int cus = num_cu();
@@ -448,6 +449,10 @@ extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     const int nChunks = ceil_div(I, kWinoKC);
     int lg = 0;
     while (lg < 5 && (panels << lg) < (5 * cus) / 8 && (nChunks >> (lg + 1)) >= 2) ++lg;
+    // A split layer that still has 32 or more stages per split (28x28, 512 -> 512): the same number
+    // of workgroups as 64-channel panels with twice the splits share each input transform between
+    // two MFMA sets (26.1 vs 27.5 us).
+    if (code == 1 && lg >= 1 && lg < 5 && O >= 64 && (nChunks >> lg) >= 32) return 2 | ((lg + 1) << 4);
     return code | (lg << 4);
 }
 
