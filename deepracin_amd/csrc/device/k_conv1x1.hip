@@ -112,14 +112,95 @@ conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, c
     }
 }
 
+// Small layers (14x14 and 28x28 maps): a 32x32 tile with 512 input channels is 256 MFMAs in a row on
+// one CU while most of the chip idles.  This form works on 16-channel x 16-pixel tiles with
+// v_mfma_f32_16x16x4_f32 (A: lane -> row lane%16, k = lane/16; B: lane -> col lane%16, k = lane/16;
+// D: lane -> col lane%16, register r -> row 4*(lane/16) + r), four times as many workgroups and a
+// quarter of the dependent MFMA chain each.  KW waves (1..16) take the 4-channel k-steps round-robin
+// in chunks of 8, the next chunk always in flight; k-steps past the end are multiplied as zeros
+// (32 cycles each) so that the loop has no branch and the compiler can count the loads.
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+constexpr int kC1Chunk = 8;         // k-steps per chunk (16 in flight was measured slower)
+constexpr int kC1Pad16 = 17;
+
+__global__ void __launch_bounds__(1024)
+conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
+                      float* __restrict__ out, int P, int I, int O, int nPT, int relu) {
+    extern __shared__ float part[];                 // [KW][16][kC1Pad16]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int KW = blockDim.x >> 6;
+    const int l16 = lane & 15, lk = lane >> 4;
+    const int o0 = (blockIdx.x / nPT) * 16, p0 = (blockIdx.x % nPT) * 16;
+    const int nK = (I + 3) / 4;                     // k-steps of 4 channels
+    const int oL = min(o0 + l16, O - 1), pL = min(p0 + l16, P - 1);
+    const bool oOk = o0 + l16 < O, pOk = p0 + l16 < P;
+
+    f32x4v acc = {0.f, 0.f, 0.f, 0.f};
+    float aA[kC1Chunk], bA[kC1Chunk], aB[kC1Chunk], bB[kC1Chunk];
+    // chunk j of this wave = its k-steps wave + KW*(8j .. 8j+7)
+    auto load_chunk = [&](float (&a)[kC1Chunk], float (&b)[kC1Chunk], int j) {
+#pragma unroll
+        for (int u = 0; u < kC1Chunk; ++u) {
+            const int c = min(4 * (wave + KW * (kC1Chunk * j + u)) + lk, I - 1);
+            a[u] = w[(size_t)c * O + oL];
+            b[u] = in[(size_t)c * P + pL];
+        }
+    };
+    auto multiply = [&](const float (&a)[kC1Chunk], const float (&b)[kC1Chunk], int j) {
+#pragma unroll
+        for (int u = 0; u < kC1Chunk; ++u) {
+            const bool cOk = 4 * (wave + KW * (kC1Chunk * j + u)) + lk < I;
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32((cOk && oOk) ? a[u] : 0.0f, (cOk && pOk) ? b[u] : 0.0f, acc, 0, 0, 0);
+        }
+    };
+    const int mine = (nK - wave + KW - 1) / KW;                 // k-steps of this wave (>= 0)
+    const int chunks = (mine + kC1Chunk - 1) / kC1Chunk;
+    // Two buffers, the next chunk always on its way.  The loop leaves right after the last real
+    // chunk: the loads issued beyond it (clamped addresses) are never waited for.
+    load_chunk(aA, bA, 0);
+    for (int j = 0; j < chunks;) {
+        load_chunk(aB, bB, j + 1);
+        multiply(aA, bA, j);
+        if (++j >= chunks) break;
+        load_chunk(aA, bA, j + 1);
+        multiply(aB, bB, j);
+        ++j;
+    }
+
+#pragma unroll
+    for (int r = 0; r < 4; ++r) part[(wave * 16 + 4 * lk + r) * kC1Pad16 + l16] = acc[r];
+    __syncthreads();
+    for (int idx = tid; idx < 16 * 16; idx += blockDim.x) {
+        const int ol = idx >> 4, pl = idx & 15;
+        const int o = o0 + ol, p = p0 + pl;
+        float s = 0.0f;
+        for (int k = 0; k < KW; ++k) s += part[(k * 16 + ol) * kC1Pad16 + pl];
+        if (o < O && p < P) {
+            if (bias) s += bias[o];
+            if (relu) s = fmaxf(s, 0.0f);
+            out[(size_t)o * P + p] = s;
+        }
+    }
+}
+
 }  // namespace drhip
 
 using namespace drhip;
 
-// Waves per output tile: as many as give every wave at least two 8-channel stages, more when the
-// layer has few tiles.  variant = number of waves (1, 2, 4, 8).
+// variant = waves per output tile (1, 2, 4, 8; 16 only with 0x100) | 0x100 for 16x16 tiles.
+// 32x32 tiles: as many waves as give every wave at least two 8-channel stages, more when the layer
+// has few tiles.  Layers with fewer 32x32 tiles than CUs take the 16x16 form with one wave per 8
+// k-steps (one chunk, a single round of loads).
 extern "C" int drhip_conv1x1_pick_variant(int P, int I, int O) {
     const int tiles = ceil_div(O, 32) * ceil_div(P, 32);
+    if (tiles < num_cu() && ceil_div(O, 16) * ceil_div(P, 16) <= 2 * num_cu()) {
+        const int nK = ceil_div(I, 4);
+        int kw = 1;
+        while (kw < 4 && nK > 8 * kw) kw *= 2;
+        if (nK > 32) kw = 8;                        // more than one chunk per wave: measured better with 8 waves
+        return 0x100 | kw;
+    }
     const int stages = ceil_div(I, kC1KC);
     int kw = 1;
     while (kw < 8 && stages >= 4 * kw && tiles * kw < 8 * num_cu()) kw *= 2;
@@ -133,6 +214,15 @@ extern "C" int drhip_conv1x1_f32(const float* in, const float* w, const float* b
     DRHIP_REQUIRE((long long)P * I < (1ll << 31) && (long long)P * O < (1ll << 31) && (long long)I * O < (1ll << 31),
                   "drhip_conv1x1_f32: tensor too large for 32-bit indexing");
     if (variant == 0) variant = drhip_conv1x1_pick_variant(P, I, O);
+    if (variant & 0x100) {
+        const int kw = variant & 0xff;
+        DRHIP_REQUIRE((variant >> 9) == 0, "drhip_conv1x1_f32: unknown variant %#x", variant);
+        DRHIP_REQUIRE(kw == 1 || kw == 2 || kw == 4 || kw == 8 || kw == 16, "drhip_conv1x1_f32: unknown variant %#x (16x16 tiles: 1..16 waves)", variant);
+        const int nPT16 = ceil_div(P, 16), nOT16 = ceil_div(O, 16);
+        launch(conv1x1_mfma16_kernel, dim3(nPT16 * nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
+               in, w, bias, out, P, I, O, nPT16, relu);
+        return launched("conv1x1_mfma16_kernel");
+    }
     DRHIP_REQUIRE(variant == 1 || variant == 2 || variant == 4 || variant == 8, "drhip_conv1x1_f32: unknown variant %d (waves per tile: 1, 2, 4, 8)", variant);
     const int nPT = ceil_div(P, 32), nOT = ceil_div(O, 32);
     const size_t ldsBytes = variant > 1 ? (size_t)variant * 32 * kC1Pad * sizeof(float) : 0;

@@ -137,7 +137,9 @@ size_t drhip_conv3x3_winograd_workspace_floats(int W, int H, int I, int O, int v
  * [I][O]->[O][I] re-layout (Kernels/dR_conv2d1x1.cl:4-53, src/dR_nodes_conv2d.c:1605-1716). */
 int drhip_conv1x1_f32(const float* in, const float* w, const float* bias, float* out,
                       int P, int I, int O, int relu, int variant, void* stream);
-/* Register-tile configuration for a 1x1 layer (replaces dR_conv2d_1x1_schedule, :1526-1602). */
+/* Tile configuration for a 1x1 layer (replaces dR_conv2d_1x1_schedule, :1526-1602): waves per
+ * output tile (1, 2, 4, 8 for 32x32 tiles; | 0x100 = 16x16 tiles, 1..16 waves, for small layers).
+ * variant 0 in drhip_conv1x1_f32 = let the launcher pick. */
 int drhip_conv1x1_pick_variant(int P, int I, int O);
 
 /* ---- pooling ----------------------------------------------------------------------------------

@@ -186,7 +186,7 @@ def test_winograd_rejects_bad_arguments(lib, dev):
     assert b"workspace" in lib.drhip_last_error()
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8, 0x101, 0x102, 0x108, 0x110])
 @pytest.mark.parametrize("P,I,O", [(3025, 128, 16), (3025, 16, 64), (196, 512, 1000), (196, 512, 64), (784, 256, 32), (50, 7, 5), (1, 1, 1), (33, 9, 65), (70, 24, 40)])
 def test_conv1x1(lib, dev, oracle, variant, P, I, O):
     x, w, b = np.abs(rnd(I, 1, P)), rnd(I, O, 1, 1, scale=np.sqrt(2.0 / I)), rnd(O, scale=0.01)
@@ -382,7 +382,7 @@ def test_conv_direct_sweep(lib, dev, oracle, W, H, I, O, kw, kh, sx, sy):
 
 
 @pytest.mark.parametrize("P,I,O,variant", _sweep(13, 20, lambda r: (
-    int(r.integers(1, 400)), int(r.integers(1, 100)), int(r.integers(1, 100)), int(r.choice([0, 1, 2, 4, 8])))))
+    int(r.integers(1, 400)), int(r.integers(1, 100)), int(r.integers(1, 100)), int(r.choice([0, 1, 2, 4, 8, 0x101, 0x104, 0x110])))))
 def test_conv1x1_sweep(lib, dev, oracle, P, I, O, variant):
     x, w, b = rnd(I, 1, P), rnd(I, O, 1, 1, scale=np.sqrt(2.0 / I)), rnd(O, scale=0.01)
     want = oracle.conv1x1(x, w, b, relu=False)
