@@ -215,6 +215,15 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
         for (int nt = 0; nt < NT; ++nt) f[nt] = buf_load4(rU, fOff + 4u * (unsigned)(nt * 32 * 8), soff);
     };
 
+    // The epilogue's bias values are fetched now: a load issued there would add a trip to memory
+    // to the tail of every workgroup.
+    constexpr bool kBiasEarly = NT <= 2;
+    float biasEarly[kBiasEarly ? OB / 8 : 1];
+    if (kBiasEarly && bias && gridDim.y == 1) {
+#pragma unroll
+        for (int q = 0; q < OB / 8; ++q) biasEarly[q] = bias[min(o0 + (tid >> 5) + 8 * q, O - 1)];
+    }
+
     f32x16 acc[4][NT];
 #pragma unroll
     for (int e = 0; e < 4; ++e)
@@ -324,7 +333,7 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
         float y10 = p[1][0] - p[2][0] + p[3][0], y11 = p[1][1] - p[2][1] + p[3][1];
         if (direct) {
             if (eTileOk && o < O) {
-                if (bias) { const float bv = bias[o]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
+                if (bias) { const float bv = kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
                 if (relu & kEpiRelu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
                 if (relu & kEpiMaxPool2)        // W, H even: the tile is one window of a 2x2/2 max pool
                     out[(size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1)] = fmaxf(fmaxf(y00, y01), fmaxf(y10, y11));
@@ -448,7 +457,8 @@ extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     const int panels = ceil_div(T, 32) * ceil_div(O, code == 2 ? 64 : 32);
     const int nChunks = ceil_div(I, kWinoKC);
     int lg = 0;
-    while (lg < 5 && (panels << lg) < (5 * cus) / 8 && (nChunks >> (lg + 1)) >= 2) ++lg;
+    // (a split costs a second kernel: below 6 stages in all it does not pay)
+    while (lg < 5 && nChunks >= 6 && (panels << lg) < (5 * cus) / 8 && (nChunks >> (lg + 1)) >= 2) ++lg;
     // A split layer that still has 32 or more stages per split (28x28, 512 -> 512): the same number
     // of workgroups as 64-channel panels with twice the splits share each input transform between
     // two MFMA sets (26.1 vs 27.5 us).
