@@ -398,4 +398,5 @@ def test_pick_variants_are_launchable(lib):
     for (W, H, I, O) in [(224, 224, 3, 64), (224, 224, 64, 64), (56, 56, 256, 256), (14, 14, 512, 512), (55, 55, 16, 64), (1, 1, 1, 1)]:
         v = lib.drhip_conv3x3_winograd_pick_variant(W, H, I, O)
         assert v >= 1
-        assert lib.drhip_conv1x1_pick_variant(W * H, I, O) in (1, 2, 4, 8)
+        c = lib.drhip_conv1x1_pick_variant(W * H, I, O)          # waves per tile | 0x100 for 16x16 tiles
+        assert (c in (1, 2, 4, 8)) or (c & 0x100 and (c & 0xff) in (1, 2, 4, 8, 16) and c >> 9 == 0)
