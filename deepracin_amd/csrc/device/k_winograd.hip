@@ -347,6 +347,192 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     }
 }
 
+
+// The same algorithm on 16-tile x 16-channel blocks with v_mfma_f32_16x16x4_f32, for layers with few
+// tiles (28x28 and 14x14 maps): four times as many workgroups as 32x32 blocks give, a quarter of
+// the dependent MFMA chain in each, so fewer (or no) input-channel splits are needed to fill the
+// chip.  Lane -> (tile lane%16, channel lane/16 of a 4-channel k-step); a stage of 8 channels is
+// two k-steps.  The filters keep their layout: lane/16 = k picks the 16-byte half (k & 1) and the
+// component pair (k >> 1) of it.  D: lane -> tile lane%16, register r -> channel 4*(lane/16) + r.
+// A workgroup owns 16 tiles x OB = 16*NB output channels.
+typedef float f32x4acc __attribute__((ext_vector_type(4)));
+
+template <int NB>
+__global__ void __launch_bounds__(kWinoThreads)
+winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ U,
+                           const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
+                           int W, int H, int I, int O, int tilesX, int T, int nTB, int nBlocks,
+                           int chunksPerSplit, int relu, int vec2) {
+    constexpr int TB = 16, OB = 16 * NB, KC = kWinoKC;
+    extern __shared__ float P[];                    // epilogue only: [4 rows][2][OB o][16 t] floats
+
+    const int perXcd = gridDim.x / kXcds;
+    const int logical = (blockIdx.x % kXcds) * perXcd + blockIdx.x / kXcds;
+    if (logical >= nBlocks) return;
+    const int o0 = (logical / nTB) * OB;
+    const int t0 = (logical % nTB) * TB;
+    const int split = blockIdx.y, nSplits = gridDim.y;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // = row of the transform
+    const int l16 = lane & 15, lk = lane >> 4;
+    const int plane = H * W;
+    const int nChunksAll = (I + KC - 1) / KC;
+    const int chBegin = split * chunksPerSplit;
+    const int chEnd = min(nChunksAll, chBegin + chunksPerSplit);
+    const int Opad = wino_opad(O);
+
+    // window rows, offsets and edge masks exactly as in the 32-tile kernel
+    const int tg = t0 + l16;
+    const bool tileOk = tg < T;
+    const int ty = tileOk ? tg / tilesX : 0, tx = tileOk ? tg % tilesX : 0;
+    const int x0 = 2 * tx - 1, y0 = 2 * ty - 1;
+    const int rowA = wave, rowB = (wave < 2) ? 2 : 1;
+    const float sgn = (wave == 1) ? 1.0f : -1.0f;
+    const bool shifted = tg == 0;
+    const int xLoad = shifted ? 0 : x0;
+    const int yaRow = y0 + rowA, ybRow = y0 + rowB;
+    const unsigned offVA = (tileOk && yaRow >= 0 && yaRow < H) ? 4u * (unsigned)(lk * plane + yaRow * W + xLoad) : kOutOfRange;
+    const unsigned offVB = (tileOk && ybRow >= 0 && ybRow < H) ? 4u * (unsigned)(lk * plane + ybRow * W + xLoad) : kOutOfRange;
+    const bool c0ok = x0 >= 0, c2ok = x0 + 2 < W, c3ok = x0 + 3 < W;
+
+    const __amdgpu_buffer_rsrc_t rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kBufferFlags);
+    auto load_rows = [&](float (&d)[8], __amdgpu_buffer_rsrc_t r, unsigned soff) {
+        const f32x4 a = buf_load4(r, offVA, soff), b = buf_load4(r, offVB, soff);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) { d[s] = a[s]; d[4 + s] = b[s]; }
+    };
+    auto load_rows_plain = [&](float (&d)[8], int cbase) { load_rows(d, rIn, 4u * (unsigned)(cbase * plane)); };
+    auto load_rows_ranged = [&](float (&d)[8], int cbase) {
+        const int left = max(I - cbase, 0);
+        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(in + (size_t)min(cbase, I) * plane), 0,
+                                                                             left * plane * 4, kBufferFlags);
+        load_rows(d, r, 0u);
+    };
+    const __amdgpu_buffer_rsrc_t rU = __builtin_amdgcn_make_buffer_rsrc((void*)U, 0, 16 * nChunksAll * Opad * 8 * 4, kBufferFlags);
+    const unsigned fOff = 4u * (unsigned)((o0 + l16) * 8 + 4 * (lk & 1));
+    const bool oddPair = (lk >> 1) != 0;            // which components of the 16 bytes: {0,2} or {1,3}
+    auto load_filters = [&](f32x4 (&f)[NB], int e, int chunk) {
+        const unsigned soff = 4u * (unsigned)(((4 * wave + e) * nChunksAll + chunk) * Opad * 8);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) f[nb] = buf_load4(rU, fOff + 4u * (unsigned)(nb * 16 * 8), soff);
+    };
+
+    float biasEarly[OB / 16];
+    if (bias && gridDim.y == 1) {
+#pragma unroll
+        for (int q = 0; q < OB / 16; ++q) biasEarly[q] = bias[min(o0 + (tid >> 4) + 16 * q, O - 1)];
+    }
+
+    f32x4acc acc[4][NB];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[e][nb] = f32x4acc{0.f, 0.f, 0.f, 0.f};
+
+    float raw[2][8];
+    f32x4 f[4][NB];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) load_rows_ranged(raw[ks], chBegin * KC + 4 * ks);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) load_filters(f[e], e, chBegin);
+
+    auto stage = [&](int ch, auto plainNext) {
+        const int next = min(ch + 1, nChunksAll - 1);
+        float b[2][4];                              // [k-step][xi within the row]
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            float m[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) m[s] = fmaf(sgn, raw[ks][4 + s], raw[ks][s]);
+            const float s1 = shifted ? m[0] : m[1], s2 = shifted ? m[1] : m[2], s3 = shifted ? m[2] : m[3];
+            m[0] = c0ok ? m[0] : 0.0f;
+            m[1] = s1;
+            m[2] = c2ok ? s2 : 0.0f;
+            m[3] = c3ok ? s3 : 0.0f;
+            b[ks][0] = m[0] - m[2];
+            b[ks][1] = m[1] + m[2];
+            b[ks][2] = m[2] - m[1];
+            b[ks][3] = m[3] - m[1];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int eg = 0; eg < 2; ++eg) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+                for (int e = 2 * eg; e < 2 * eg + 2; ++e)
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) {
+                        const float a = oddPair ? f[e][nb][2 * ks + 1] : f[e][nb][2 * ks];
+                        acc[e][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ks][e], acc[e][nb], 0, 0, 0);
+                    }
+                if (eg == 0) {
+                    if constexpr (decltype(plainNext)::value) load_rows_plain(raw[ks], (ch + 1) * KC + 4 * ks);
+                    else load_rows_ranged(raw[ks], (ch + 1) * KC + 4 * ks);
+                } else {
+                    load_filters(f[ks], ks, next);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        load_filters(f[2], 2, next);
+        load_filters(f[3], 3, next);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    const int chMain = max(chBegin, min(chEnd, I / KC - 1));
+    int ch = chBegin;
+    for (; ch < chMain; ++ch) stage(ch, std::true_type{});
+    for (; ch < chEnd; ++ch) stage(ch, std::false_type{});
+
+    // ---- epilogue: right factor in registers, rows meet in LDS, left factor, bias, ReLU, store ----
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float m0 = acc[0][nb][r], m1 = acc[1][nb][r], m2 = acc[2][nb][r], m3 = acc[3][nb][r];
+            const int ol = 16 * nb + 4 * lk + r;
+            P[((wave * 2 + 0) * OB + ol) * TB + l16] = m0 + m1 + m2;
+            P[((wave * 2 + 1) * OB + ol) * TB + l16] = m1 - m2 + m3;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+
+    const bool direct = nSplits == 1;
+    const int et = tid & 15, eo = tid >> 4;
+    const int etg = t0 + et;
+    const bool eTileOk = etg < T;
+    const int ox = eTileOk ? 2 * (etg % tilesX) : 0, oy = eTileOk ? 2 * (etg / tilesX) : 0;
+    f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
+#pragma unroll
+    for (int q = 0; q < OB / 16; ++q) {
+        const int ol = eo + 16 * q, o = o0 + ol;
+        float p[4][2];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            p[r][0] = P[((r * 2 + 0) * OB + ol) * TB + et];
+            p[r][1] = P[((r * 2 + 1) * OB + ol) * TB + et];
+        }
+        float y00 = p[0][0] + p[1][0] + p[2][0], y01 = p[0][1] + p[1][1] + p[2][1];
+        float y10 = p[1][0] - p[2][0] + p[3][0], y11 = p[1][1] - p[2][1] + p[3][1];
+        if (direct) {
+            if (eTileOk && o < O) {
+                if (bias) { const float bv = biasEarly[q]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
+                if (relu & kEpiRelu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
+                if (relu & kEpiMaxPool2)
+                    out[(size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1)] = fmaxf(fmaxf(y00, y01), fmaxf(y10, y11));
+                else
+                    wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, y00, y01, y10, y11);
+            }
+        } else {
+            f32x4 v = {y00, y01, y10, y11};
+            wsTiles[(size_t)ol * TB + et] = v;
+        }
+    }
+}
+
 // out[o][2x2 tile] = act(bias[o] + sum over splits of the partial tile), splits added in order.
 // One lane per (o, tile); partials are [split][panel][o in panel][tile in panel] float4.
 // Workgroup b works for panel (b % 8) * perXcd + ..., i.e. on the XCD whose workgroups wrote that
@@ -387,12 +573,14 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
 
 // variant = output channels per workgroup (low 4 bits: 1 -> 32, 2 -> 64, 3 -> 128)
 //         | log2(number of input-channel splits) << 4
-struct WinoCfg { int nt, splits; };
+//         | 0x100: 16-tile blocks (then the low 4 bits mean 1 -> 16, 2 -> 32, 3 -> 64 channels)
+struct WinoCfg { int nt, splits, tb; };
 
 static bool wino_variant(int variant, WinoCfg* c) {
     const int lg = (variant >> 4) & 0xf;
-    if (lg > 6 || (variant >> 8)) return false;
+    if (lg > 6 || (variant >> 9)) return false;
     c->splits = 1 << lg;
+    c->tb = (variant & 0x100) ? 16 : 32;
     switch (variant & 0xf) {
         case 1: c->nt = 1; return true;
         case 2: c->nt = 2; return true;
@@ -407,8 +595,8 @@ static WinoGeom wino_geom(int W, int H, int I, int O, const WinoCfg& c) {
     WinoGeom g;
     g.tilesX = (W + 1) / 2;
     g.T = g.tilesX * ((H + 1) / 2);
-    g.nTB = ceil_div(g.T, 32);
-    g.nOB = ceil_div(O, 32 * c.nt);
+    g.nTB = ceil_div(g.T, c.tb);
+    g.nOB = ceil_div(O, c.tb * c.nt);
     g.nBlocks = g.nTB * g.nOB;
     g.nChunks = ceil_div(I, kWinoKC);
     int splits = c.splits < g.nChunks ? c.splits : g.nChunks;
@@ -419,17 +607,20 @@ static WinoGeom wino_geom(int W, int H, int I, int O, const WinoCfg& c) {
 
 // Workspace: [splits][panel][o in panel][tile in panel] partial 2x2 tiles (float4 each).
 
-template <int NT>
+template <int NT, int TB>
 static int launch_wino(const float* in, const float* U, const float* bias, float* out, float* workspace,
                        int W, int H, int I, int O, int relu, const WinoCfg& c, hipStream_t s) {
-    constexpr int TB = 32, OB = 32 * NT;
+    constexpr int OB = TB * NT;
     const WinoGeom g = wino_geom(W, H, I, O, c);
     const int gridX = ceil_div(g.nBlocks, kXcds) * kXcds;
     const size_t ldsBytes = 4 * 2 * OB * TB * sizeof(float);
     const int vec2 = ((W & 1) == 0) && (((size_t)out & 7) == 0);
-    launch((winograd_f23_mfma_kernel<NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
-                       in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks,
-                       g.chunksPerSplit, relu, vec2);
+    if constexpr (TB == 32)
+        launch((winograd_f23_mfma_kernel<NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
+               in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
+    else
+        launch((winograd_f23_mfma16_kernel<NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
+               in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
     if (g.splits > 1) {
         const int perXcd = gridX / kXcds;
@@ -449,10 +640,15 @@ using namespace drhip;
 //     the panels alone give several workgroups per CU and sharing the input transform pays;
 //   - the input channels are split until at least ~160 workgroups exist, keeping at least 2 stages
 //     of 8 channels per split;
-//   - split layers with very long channel loops trade panel width against split count.
+//   - split layers with very long channel loops trade panel width against split count;
+//   - small layers take the 16-tile kernel.
 extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     const int T = ((W + 1) / 2) * ((H + 1) / 2);
     const int cus = num_cu();
+    // Small layers (SqueezeNet's expand convolutions: <= 8 stages, a few dozen 32x32 panels) are bound
+    // by the latency of one workgroup, not by throughput: 16x16 blocks, unsplit, one launch
+    // (in a replayed launch graph 4.2-5.8 us per layer against 5.1-7.1 us for the 32x32 forms).
+    if (ceil_div(T, 32) * ceil_div(O, 32) < cus / 2 && ceil_div(I, kWinoKC) <= 16) return 0x101;
     const int code = (O > 32 && T >= 8192) ? 2 : 1;
     const int panels = ceil_div(T, 32) * ceil_div(O, code == 2 ? 64 : 32);
     const int nChunks = ceil_div(I, kWinoKC);
@@ -476,7 +672,7 @@ extern "C" size_t drhip_conv3x3_winograd_workspace_floats(int W, int H, int I, i
     if (W <= 0 || H <= 0 || I <= 0 || O <= 0 || !wino_variant(variant, &c)) return 0;
     const WinoGeom g = wino_geom(W, H, I, O, c);
     if (g.splits <= 1) return 0;
-    return (size_t)g.splits * g.nBlocks * (32 * c.nt) * 32 * 4;
+    return (size_t)g.splits * g.nBlocks * (c.tb * c.nt) * c.tb * 4;
 }
 
 extern "C" int drhip_winograd_filter_transform_f32(const float* w, float* U, int I, int O, void* stream) {
@@ -508,7 +704,12 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
     DRHIP_REQUIRE(g.splits == 1 || workspace, "drhip_conv3x3_winograd_f32: variant %d splits the input channels and needs a workspace", variant);
     DRHIP_REQUIRE(g.splits <= 65535, "drhip_conv3x3_winograd_f32: too many input-channel splits");
     hipStream_t s = as_stream(stream);
-    if (c.nt == 1) return launch_wino<1>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
-    if (c.nt == 2) return launch_wino<2>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
-    return launch_wino<4>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
+    if (c.tb == 16) {
+        if (c.nt == 1) return launch_wino<1, 16>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
+        if (c.nt == 2) return launch_wino<2, 16>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
+        return launch_wino<4, 16>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
+    }
+    if (c.nt == 1) return launch_wino<1, 32>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
+    if (c.nt == 2) return launch_wino<2, 32>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
+    return launch_wino<4, 32>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);
 }

@@ -111,7 +111,7 @@ def test_winograd_filter_transform(lib, dev, oracle):
     assert np.allclose(got, expect, rtol=1e-6, atol=1e-7)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 0x11, 0x21, 0x12, 0x33])
+@pytest.mark.parametrize("variant", [1, 2, 3, 0x11, 0x21, 0x12, 0x33, 0x101, 0x102, 0x103, 0x111, 0x122])
 @pytest.mark.parametrize("W,H,I,O", [
     (56, 56, 64, 64),        # config 1
     (55, 55, 16, 64),        # fire expand3x3: odd size, two stages of 8 channels
@@ -137,7 +137,7 @@ def test_winograd_conv(lib, dev, oracle, variant, W, H, I, O):
     assert rel_err(dev.get(out, want2.shape), want2) <= TOL
 
 
-@pytest.mark.parametrize("variant", [1, 2, 0x11, 0x22])
+@pytest.mark.parametrize("variant", [1, 2, 0x11, 0x22, 0x101, 0x112])
 @pytest.mark.parametrize("W,H,I,O", [(56, 56, 64, 64), (28, 12, 24, 40), (2, 2, 1, 1), (224, 224, 3, 64)])
 def test_winograd_fused_maxpool(lib, dev, oracle, variant, W, H, I, O):
     """Epilogue flag 2: the kernel stores the 2x2/2 maximum of every output tile -- bit for bit what
@@ -353,7 +353,7 @@ def _sweep(seed, count, draw):
 
 @pytest.mark.parametrize("W,H,I,O,variant", _sweep(11, 24, lambda r: (
     int(r.integers(1, 41)), int(r.integers(1, 41)), int(r.integers(1, 41)), int(r.integers(1, 71)),
-    int(r.choice([0, 1, 2, 3, 0x11, 0x12, 0x21, 0x31]))))
+    int(r.choice([0, 1, 2, 3, 0x11, 0x12, 0x21, 0x31, 0x101, 0x102, 0x103, 0x111, 0x121]))))
     + [(1, 37, 9, 31, 0x11), (37, 1, 8, 32, 1), (3, 3, 64, 33, 0x21), (40, 2, 17, 1, 2)])
 def test_winograd_sweep(lib, dev, oracle, W, H, I, O, variant):
     x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
