@@ -56,6 +56,42 @@ pool_kernel(const float* __restrict__ in, float* __restrict__ out, int* __restri
     }
 }
 
+// 2x2 and 3x3 windows inside one channel (sz = 1): the same scan, but all samples are fetched
+// first, unconditionally and from clamped positions, so a lane pays one trip to memory instead of
+// one per sample; samples outside the image become 0.0f by select afterwards.
+template <bool MAX, bool ARG, int SX, int SY>
+__global__ void __launch_bounds__(256)
+pool_small_kernel(const float* __restrict__ in, float* __restrict__ out, int* __restrict__ argmax,
+                  int W, int H, int C, int Wo, int Ho, int stx, int sty, int stz) {
+    const int total = Wo * Ho * ((C + stz - 1) / stz);
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int xo = idx % Wo, yo = (idx / Wo) % Ho, zo = idx / (Wo * Ho);
+    const int x0 = xo * stx, y0 = yo * sty, z = zo * stz;
+    const float* pc = in + (size_t)z * H * W;
+    float v[SY][SX];
+#pragma unroll
+    for (int dy = 0; dy < SY; ++dy)
+#pragma unroll
+        for (int dx = 0; dx < SX; ++dx) v[dy][dx] = pc[min(y0 + dy, H - 1) * W + min(x0 + dx, W - 1)];
+    float r = MAX ? -FLT_MAX : 0.0f;
+    int where = -1;
+#pragma unroll
+    for (int dy = 0; dy < SY; ++dy)
+#pragma unroll
+        for (int dx = 0; dx < SX; ++dx) {
+            const bool inside = x0 + dx < W && y0 + dy < H;
+            const float s = inside ? v[dy][dx] : 0.0f;
+            if (MAX) {
+                if (s > r) { r = s; if (ARG) where = inside ? (z * H + y0 + dy) * W + x0 + dx : -1; }
+            } else {
+                r += s;
+            }
+        }
+    out[idx] = MAX ? r : r / (float)(SX * SY);
+    if (MAX && ARG) argmax[idx] = where;
+}
+
 template <bool MAX, bool ARG>
 __global__ void __launch_bounds__(256)
 pool_wave_kernel(const float* __restrict__ in, float* __restrict__ out, int* __restrict__ argmax,
@@ -69,16 +105,29 @@ pool_wave_kernel(const float* __restrict__ in, float* __restrict__ out, int* __r
     const int x0 = xo * stx, y0 = yo * sty, z0 = zo * stz;
     float r = MAX ? -FLT_MAX : 0.0f;
     int pos = 0x7fffffff, where = -1;                // scan position and flat index of the running maximum
-    for (int e = lane; e < n; e += 64) {
-        const int dx = e % sx, dy = (e / sx) % sy, dz = e / (sx * sy);
-        const int x = x0 + dx, y = y0 + dy, z = z0 + dz;
-        const bool inside = x < W && y < H && z < C;
-        const int flat = (z * H + y) * W + x;
-        const float v = inside ? in[flat] : 0.0f;
-        if (MAX) {
-            if (v > r) { r = v; pos = e; where = inside ? flat : -1; }
-        } else {
-            r += v;
+    // four samples per lane and round, fetched unconditionally from clamped positions
+    for (int e0 = lane; e0 < n; e0 += 256) {
+        float v[4]; int flat[4]; bool inside[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = e0 + 64 * u;
+            const int dx = e % sx, dy = (e / sx) % sy, dz = e / (sx * sy);
+            const int x = x0 + dx, y = y0 + dy, z = z0 + dz;
+            inside[u] = e < n && x < W && y < H && z < C;
+            flat[u] = (z * H + y) * W + x;
+            v[u] = in[(min(z, C - 1) * H + min(y, H - 1)) * W + min(x, W - 1)];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = e0 + 64 * u;
+            if (e < n) {
+                const float s = inside[u] ? v[u] : 0.0f;
+                if (MAX) {
+                    if (s > r) { r = s; pos = e; where = inside[u] ? flat[u] : -1; }
+                } else {
+                    r += s;
+                }
+            }
         }
     }
 #pragma unroll
@@ -125,6 +174,22 @@ extern "C" int drhip_pool_f32(const float* in, float* out, int* argmax_out,
         else
             launch((pool_wave_kernel<false, false>), dim3(wblocks), dim3(block), 0, s, in, out, (int*)nullptr, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
         return launched("pool_wave_kernel");
+    }
+    if (sz == 1 && sx == sy && (sx == 2 || sx == 3)) {
+        const dim3 g((unsigned)((total + block - 1) / block)), b(block);
+        int* none = nullptr;
+#define DRHIP_POOL_SMALL(MAXV, ARGV, S, ARGP) launch((pool_small_kernel<MAXV, ARGV, S, S>), g, b, 0, s, in, out, ARGP, W, H, C, Wo, Ho, stx, sty, stz)
+        if (sx == 2) {
+            if (type == 0 && argmax_out) DRHIP_POOL_SMALL(true, true, 2, argmax_out);
+            else if (type == 0) DRHIP_POOL_SMALL(true, false, 2, none);
+            else DRHIP_POOL_SMALL(false, false, 2, none);
+        } else {
+            if (type == 0 && argmax_out) DRHIP_POOL_SMALL(true, true, 3, argmax_out);
+            else if (type == 0) DRHIP_POOL_SMALL(true, false, 3, none);
+            else DRHIP_POOL_SMALL(false, false, 3, none);
+        }
+#undef DRHIP_POOL_SMALL
+        return launched("pool_small_kernel");
     }
     if (type == 0 && argmax_out)
         launch((pool_kernel<true, true>), dim3(blocks), dim3(block), 0, s, in, out, argmax_out, W, H, C, Wo, Ho, Co, sx, sy, sz, stx, sty, stz);
