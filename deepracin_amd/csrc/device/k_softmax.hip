@@ -1,5 +1,6 @@
-// Softmax over a flat fp32 vector in ONE workgroup: wavefront-level butterfly reductions
-// (ds_bpermute via __shfl_xor) for max and sum, one small LDS exchange between the waves.
+// Softmax over a flat fp32 vector in ONE workgroup of four waves: wavefront-level butterfly
+// reductions (ds_bpermute via __shfl_xor) for max and sum, one small LDS exchange between the waves;
+// vectors of up to 2048 elements are read once and kept in registers.
 //
 // The reference computes exp(x) on the device, downloads the vector, sums it sequentially on the
 // host and launches a scale kernel (src/dR_nodes_math.c:620-678).  Mathematically this kernel is
@@ -11,7 +12,8 @@
 
 namespace drhip {
 
-constexpr int kSoftmaxThreads = 1024;
+constexpr int kSoftmaxThreads = 256;
+constexpr int kSoftmaxRegs = 8;     // vectors of up to 2048 elements live in registers: one read of x
 
 __device__ inline float wave_max(float v) {
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
@@ -22,15 +24,58 @@ __device__ inline float wave_sum(float v) {
     return v;
 }
 
+// Workgroup-wide maximum / sum; the result is valid in every lane.  `red` has one slot per wave.
+template <bool MAX>
+__device__ inline float block_reduce(float v, float* red) {
+    constexpr int nwaves = kSoftmaxThreads / kWave;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    v = MAX ? wave_max(v) : wave_sum(v);
+    __syncthreads();                    // red may still be read from the previous reduction
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+#pragma unroll
+    for (int w = 1; w < nwaves; ++w) r = MAX ? fmaxf(r, red[w]) : r + red[w];
+    return r;
+}
+
 // xdef.partials != NULL: the logits arrive as the partial sums of the GEMV in front (slices added
-// in order, then its bias and ReLU); they are finished into y first (and into xdef.finished, when
-// the caller wants to read the logits too), which then serves as x.
+// in order, then its bias and ReLU); they are finished first (and stored to xdef.finished when the
+// caller wants to read the logits too).
+template <bool SMALL>
 __global__ void __launch_bounds__(kSoftmaxThreads)
 softmax_kernel(const float* x, drhip_deferred_vec xdef, float* y, int n) {     // no __restrict__: x may become y
     __shared__ float red[kSoftmaxThreads / kWave];
-    __shared__ float bcast;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    constexpr int nwaves = kSoftmaxThreads / kWave;
+    const int tid = threadIdx.x;
+    if (SMALL) {                                    // n <= kSoftmaxThreads * kSoftmaxRegs
+        float v[kSoftmaxRegs];
+#pragma unroll
+        for (int u = 0; u < kSoftmaxRegs; ++u) {
+            const int i = tid + u * kSoftmaxThreads;
+            v[u] = -FLT_MAX;
+            if (i < n) {
+                v[u] = xdef.partials ? deferred_element(xdef, i) : x[i];
+                if (xdef.partials && xdef.finished) xdef.finished[i] = v[u];
+            }
+        }
+        float m = -FLT_MAX;
+#pragma unroll
+        for (int u = 0; u < kSoftmaxRegs; ++u) m = fmaxf(m, v[u]);
+        m = block_reduce<true>(m, red);
+        float s = 0.0f;
+#pragma unroll
+        for (int u = 0; u < kSoftmaxRegs; ++u) {
+            v[u] = (tid + u * kSoftmaxThreads < n) ? expf(v[u] - m) : 0.0f;
+            s += v[u];
+        }
+        const float inv = 1.0f / block_reduce<false>(s, red);
+#pragma unroll
+        for (int u = 0; u < kSoftmaxRegs; ++u) {
+            const int i = tid + u * kSoftmaxThreads;
+            if (i < n) y[i] = v[u] * inv;
+        }
+        return;
+    }
     if (xdef.partials) {
         for (int i = tid; i < n; i += kSoftmaxThreads) {
             const float s = deferred_element(xdef, i);
@@ -39,33 +84,12 @@ softmax_kernel(const float* x, drhip_deferred_vec xdef, float* y, int n) {     /
         }
         x = y;
     }
-
     float m = -FLT_MAX;
     for (int i = tid; i < n; i += kSoftmaxThreads) m = fmaxf(m, x[i]);
-    m = wave_max(m);
-    if (lane == 0) red[wave] = m;
-    __syncthreads();
-    if (wave == 0) {
-        float v = lane < nwaves ? red[lane] : -FLT_MAX;
-        v = wave_max(v);
-        if (lane == 0) bcast = v;
-    }
-    __syncthreads();
-    m = bcast;
-
+    m = block_reduce<true>(m, red);
     float s = 0.0f;
     for (int i = tid; i < n; i += kSoftmaxThreads) s += expf(x[i] - m);
-    s = wave_sum(s);
-    __syncthreads();            // everyone has read bcast / red from the first round
-    if (lane == 0) red[wave] = s;
-    __syncthreads();
-    if (wave == 0) {
-        float v = lane < nwaves ? red[lane] : 0.0f;
-        v = wave_sum(v);
-        if (lane == 0) bcast = 1.0f / v;
-    }
-    __syncthreads();
-    const float inv = bcast;
+    const float inv = 1.0f / block_reduce<false>(s, red);
     for (int i = tid; i < n; i += kSoftmaxThreads) y[i] = expf(x[i] - m) * inv;
 }
 
@@ -79,7 +103,10 @@ extern "C" int drhip_softmax_ex_f32(const float* x, const drhip_deferred_vec* xd
     DRHIP_REQUIRE(!xdef || (xdef->partials && xdef->slices > 0 && xdef->n == n), "drhip_softmax_f32: deferred input must carry partial sums of a vector of length %d", n);
     DRHIP_REQUIRE(!xdef || xdef->finished != y, "drhip_softmax_f32: the finished logits and the probabilities need separate arrays");
     const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0, nullptr};
-    launch(softmax_kernel, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, xdef ? *xdef : none, y, n);
+    if (n <= kSoftmaxThreads * kSoftmaxRegs)
+        launch(softmax_kernel<true>, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, xdef ? *xdef : none, y, n);
+    else
+        launch(softmax_kernel<false>, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, xdef ? *xdef : none, y, n);
     return launched("softmax_kernel");
 }
 

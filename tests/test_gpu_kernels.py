@@ -251,10 +251,11 @@ class DeferredVec(ctypes.Structure):
     _fields_ = [("partials", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("slices", ctypes.c_int), ("n", ctypes.c_int), ("relu", ctypes.c_int), ("finished", ctypes.c_void_p)]
 
 
-def test_fc_chain_without_finishing_kernels(lib, dev, oracle):
+@pytest.mark.parametrize("N2", [1000, 2500])        # softmax with the vector in registers / re-read from memory
+def test_fc_chain_without_finishing_kernels(lib, dev, oracle, N2):
     """FC -> FC -> softmax where each consumer sums the producer's split-K partials itself: every
     result equals the one of the three separate calls bit for bit."""
-    K, N1, N2 = 1024, 2048, 1000
+    K, N1 = 1024, 2048
     x, W1, b1 = np.abs(rnd(K)), rnd(K, N1, scale=np.sqrt(2.0 / K)), rnd(N1, scale=0.01)
     W2, b2 = rnd(N1, N2, scale=np.sqrt(2.0 / N1)), rnd(N2, scale=0.01)
     xd, W1d, b1d, W2d, b2d = dev.put(x), dev.put(W1), dev.put(b1), dev.put(W2), dev.put(b2)
@@ -315,7 +316,7 @@ def test_normalize(lib, dev, oracle, C, H, W):
 
 
 def test_softmax(lib, dev, oracle):
-    for n, scale in [(1000, 3.0), (10, 1.0), (5000, 5.0), (1, 1.0)]:
+    for n, scale in [(1000, 3.0), (10, 1.0), (5000, 5.0), (1, 1.0), (2048, 2.0), (2049, 2.0), (257, 1.0)]:
         x = rnd(n, scale=scale)
         y = dev.empty(n)
         ok(lib, lib.drhip_softmax_f32(dev.put(x), y, n, None))
