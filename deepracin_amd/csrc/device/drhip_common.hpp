@@ -80,16 +80,16 @@ __device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {
 #pragma unroll
         for (int u = 0; u < 32; ++u) s += v[u];
     }
-    for (; sl + 8 <= d.slices; sl += 8) {
+    for (; sl < d.slices; sl += 8) {                // the ragged end too: clamped loads, zeros by select
         float v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = pp[(size_t)(sl + u) * d.n];
+        for (int u = 0; u < 8; ++u) v[u] = pp[(size_t)min(sl + u, d.slices - 1) * d.n];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) s += v[u];
+        for (int u = 0; u < 8; ++u) s = (sl + u < d.slices) ? s + v[u] : s;
     }
-    for (; sl < d.slices; ++sl) s += pp[(size_t)sl * d.n];
     if (d.bias) s += d.bias[row];
     if (d.relu) s = fmaxf(s, 0.0f);
+    if (d.divisor != 0.0f) s = s / d.divisor;
     return s;
 }
 

@@ -35,7 +35,7 @@ constexpr int kC1Pad = 33;          // LDS row pitch of a partial tile (floats)
 
 __global__ void __launch_bounds__(512)
 conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
-                    float* __restrict__ out, int P, int I, int O, int nPT, int relu) {
+                    float* __restrict__ out, float* __restrict__ poolPartials, int P, int I, int O, int nPT, int relu) {
     extern __shared__ float part[];                 // [KW][32][kC1Pad], used only when KW > 1
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -104,9 +104,16 @@ conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, c
         const int o = o0 + ol, p = p0 + pl;
         float s = 0.0f;
         for (int k = 0; k < KW; ++k) s += part[(k * 32 + ol) * kC1Pad + pl];
-        if (o < O && p < P) {
-            if (bias) s += bias[o];
-            if (relu) s = fmaxf(s, 0.0f);
+        if (bias && o < O) s += bias[o];
+        if (relu) s = fmaxf(s, 0.0f);
+        if (poolPartials) {
+            // sum over the tile's pixels: the 32 lanes of a half wave hold one channel (the trip count
+            // of this loop is the same for every lane, so all of them take part in the shuffles)
+            s = p < P ? s : 0.0f;
+#pragma unroll
+            for (int m = 16; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+            if (pl == 0 && o < O) poolPartials[(size_t)(p0 >> 5) * O + o] = s;
+        } else if (o < O && p < P) {
             out[(size_t)o * P + p] = s;
         }
     }
@@ -227,6 +234,24 @@ extern "C" int drhip_conv1x1_f32(const float* in, const float* w, const float* b
     const int nPT = ceil_div(P, 32), nOT = ceil_div(O, 32);
     const size_t ldsBytes = variant > 1 ? (size_t)variant * 32 * kC1Pad * sizeof(float) : 0;
     launch(conv1x1_mfma_kernel, dim3(nPT * nOT), dim3(64 * variant), ldsBytes, as_stream(stream),
-                       in, w, bias, out, P, I, O, nPT, relu);
+                       in, w, bias, out, (float*)nullptr, P, I, O, nPT, relu);
+    return launched("conv1x1_mfma_kernel");
+}
+
+extern "C" int drhip_conv1x1_poolsum_slices(int P) { return P > 0 ? ceil_div(P, 32) : 0; }
+
+extern "C" int drhip_conv1x1_poolsum_f32(const float* in, const float* w, const float* bias, float* partials,
+                                         int P, int I, int O, int relu, void* stream) {
+    DRHIP_REQUIRE(in && w && partials, "drhip_conv1x1_poolsum_f32: NULL tensor");
+    DRHIP_REQUIRE(P > 0 && I > 0 && O > 0, "drhip_conv1x1_poolsum_f32: bad shape P=%d I=%d O=%d", P, I, O);
+    DRHIP_REQUIRE((long long)P * I < (1ll << 31) && (long long)P * O < (1ll << 31) && (long long)I * O < (1ll << 31),
+                  "drhip_conv1x1_poolsum_f32: tensor too large for 32-bit indexing");
+    // 32x32 tiles with at least two waves: the pixel sums are taken where the waves' partial tiles meet
+    const int tiles = ceil_div(O, 32) * ceil_div(P, 32), stages = ceil_div(I, kC1KC);
+    int kw = 2;
+    while (kw < 8 && stages >= 4 * kw && tiles * kw < 8 * num_cu()) kw *= 2;
+    const int nPT = ceil_div(P, 32), nOT = ceil_div(O, 32);
+    launch(conv1x1_mfma_kernel, dim3(nPT * nOT), dim3(64 * kw), (size_t)kw * 32 * kC1Pad * sizeof(float), as_stream(stream),
+           in, w, bias, (float*)nullptr, partials, P, I, O, nPT, relu);
     return launched("conv1x1_mfma_kernel");
 }

@@ -225,7 +225,7 @@ extern "C" int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, c
     DRHIP_REQUIRE(p.slices <= 65535, "drhip_fc_f32: too many row slices");
     dim3 grid(p.panels, p.slices);
     hipStream_t s = as_stream(stream);
-    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0, nullptr};
+    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0, nullptr, 0.0f};
     const drhip_deferred_vec& xd = xdef ? *xdef : none;
     if (p.vec == 4) launch_gemv<4>(xdef != nullptr, grid, s, x, xd, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu, defer);
     else if (p.vec == 2) launch_gemv<2>(xdef != nullptr, grid, s, x, xd, Wt, bias, y, partials, K, N, p.rowsPerSlice, relu, defer);

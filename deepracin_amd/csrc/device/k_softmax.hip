@@ -102,7 +102,7 @@ extern "C" int drhip_softmax_ex_f32(const float* x, const drhip_deferred_vec* xd
     DRHIP_REQUIRE(n > 0, "drhip_softmax_f32: n = %d", n);
     DRHIP_REQUIRE(!xdef || (xdef->partials && xdef->slices > 0 && xdef->n == n), "drhip_softmax_f32: deferred input must carry partial sums of a vector of length %d", n);
     DRHIP_REQUIRE(!xdef || xdef->finished != y, "drhip_softmax_f32: the finished logits and the probabilities need separate arrays");
-    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0, nullptr};
+    const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0, nullptr, 0.0f};
     if (n <= kSoftmaxThreads * kSoftmaxRegs)
         launch(softmax_kernel<true>, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, xdef ? *xdef : none, y, n);
     else

@@ -112,6 +112,8 @@ gboolean conv_allocate(dR_Graph* net, dR_Node* node) {
     if (launch_has_bias(c)) ok = ok && dR_createFloatBuffer(net, &c->biasBuf, O, CL_MEM_READ_ONLY);
     const size_t ws = wino ? drhip_conv3x3_winograd_workspace_floats(c->ishape.s0, c->ishape.s1, c->shape.s2, O, c->variant) : 0;
     if (ws > 0) ok = ok && dR_createFloatBuffer(net, &c->workspaceBuf, (gint)ws, CL_MEM_READ_WRITE);   // split-K partial tiles
+    if (c->drFusedAvgPool)                      // per-tile pixel sums for the pooling behind this layer
+        ok = ok && dR_createFloatBuffer(net, &c->workspaceBuf, drhip_conv1x1_poolsum_slices(c->ishape.s0 * c->ishape.s1) * O, CL_MEM_READ_WRITE);
     return ok;
 }
 
@@ -179,7 +181,10 @@ gboolean conv_compute(dR_Graph* net, dR_Node* node) {
                                             c->variant, (float*)c->workspaceBuf, stream_of(net));
             break;
         case drConv1x1Gemm:
-            rc = drhip_conv1x1_f32(in, w, b, out, W * H, I, O, relu, c->variant, stream_of(net));
+            if (c->drFusedAvgPool)
+                rc = drhip_conv1x1_poolsum_f32(in, w, b, (float*)c->workspaceBuf, W * H, I, O, relu, stream_of(net));
+            else
+                rc = drhip_conv1x1_f32(in, w, b, out, W * H, I, O, relu, c->variant, stream_of(net));
             break;
         default:
             rc = drhip_conv2d_direct_f32(in, w, b, out, W, H, I, O, c->shape.s0, c->shape.s1,

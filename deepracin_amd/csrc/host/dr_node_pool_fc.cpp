@@ -145,16 +145,31 @@ gboolean fc_fill(dR_Graph* net, dR_Node* node) {
     return ok;
 }
 
-// Where an FC node that skipped its finishing kernel left its output.
+// Where a node that skipped its finishing kernel left its output: an FC node its slice sums, a
+// global average pooling behind a 1x1 convolution the convolution's per-tile pixel sums.
 drhip_deferred_vec deferred_output_of(dR_Node* producer) {
-    dR_FC_Data* p = fc_of(producer);
     drhip_deferred_vec d;
+    if (producer->type == tPooling) {
+        dR_Node* conv = first_input(producer);
+        dR_Conv2d_Data* c = (dR_Conv2d_Data*)conv->layer;
+        const int P = c->ishape.s0 * c->ishape.s1;
+        d.partials = (const float*)c->workspaceBuf;
+        d.bias = NULL;
+        d.slices = drhip_conv1x1_poolsum_slices(P);
+        d.n = c->shape.s3;
+        d.relu = 0;
+        d.finished = producer->output ? dev_out(producer) : NULL;
+        d.divisor = (float)P;
+        return d;
+    }
+    dR_FC_Data* p = fc_of(producer);
     d.partials = (const float*)p->partialsBuf;
     d.bias = p->useBias ? (const float*)p->biasBuf : NULL;
     d.slices = drhip_fc_slices(p->shape.s0, p->shape.s1);
     d.n = p->shape.s1;
     d.relu = p->activation == tReLU;
     d.finished = producer->output ? dev_out(producer) : NULL;   // the caller reads this tensor as well
+    d.divisor = 0.0f;
     return d;
 }
 

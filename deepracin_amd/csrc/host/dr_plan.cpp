@@ -86,6 +86,29 @@ dR_Node* pool_fusable_producer(const dR_Node* p) {
     return c;
 }
 
+// A global average pooling (one window = the whole map) behind a 1x1 convolution and in front of an
+// FC or softmax node: the convolution's epilogue sums its pixels per tile, the consumer adds the
+// tile sums and divides, and neither the convolution's tensor nor a pooling kernel is needed
+// (DR_FUSE_AVGPOOL=0 keeps them).  The pooled tensor may still be an output: the consumer stores it.
+dR_Node* avgpool_fusable_producer(const dR_Node* p) {
+    if (p->type != tPooling) return nullptr;
+    const char* env = getenv("DR_FUSE_AVGPOOL");
+    if (env && strcmp(env, "0") == 0) return nullptr;
+    const dR_Pooling_Data* pd = (const dR_Pooling_Data*)p->layer;
+    if (pd->poolingType != tAverage || pd->shape.s3 != 1 || pd->stride.s3 != 1) return nullptr;
+    if (pd->shape.s1 != pd->ishape.s0 || pd->shape.s2 != pd->ishape.s1) return nullptr;
+    if (pd->stride.s1 < pd->ishape.s0 || pd->stride.s2 < pd->ishape.s1) return nullptr;
+    if (p->outputBuf || !p->next_layers || p->next_layers->length != 1) return nullptr;
+    const dR_Node* consumer = nodes_of(p->next_layers)[0];
+    if (consumer->type != tFullyConnected && consumer->type != tSoftmax) return nullptr;
+    std::vector<dR_Node*> ins = nodes_of(p->previous_layers);
+    if (ins.size() != 1) return nullptr;
+    dR_Node* c = ins[0];
+    if (c->type != tConv2d || ((const dR_Conv2d_Data*)c->layer)->algo != drConv1x1Gemm) return nullptr;
+    if (c->output || c->outputBuf || !c->next_layers || c->next_layers->length != 1) return nullptr;
+    return c;
+}
+
 }  // namespace
 
 extern "C" {
@@ -220,12 +243,20 @@ gboolean dR_planBuffers(dR_Graph* net) {
     }
     for (dR_Node* n : sched)
         if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drAbsorbed1x1 = ((dR_Conv2d_Data*)n->layer)->drAbsorbedBy = nullptr;
+    for (dR_Node* n : sched)
+        if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drFusedPool = ((dR_Conv2d_Data*)n->layer)->drFusedAvgPool = FALSE;
     for (dR_Node* n : sched) {
-        if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drFusedPool = FALSE;
         if (n->type == tPooling) {
             dR_Node* c = pool_fusable_producer(n);
             ((dR_Pooling_Data*)n->layer)->drFused = c != nullptr;
             if (c) { ((dR_Conv2d_Data*)c->layer)->drFusedPool = TRUE; parent[c] = std::make_pair(n, 0); }
+            else if ((c = avgpool_fusable_producer(n)) != nullptr) {
+                dR_Node* consumer = nodes_of(n->next_layers)[0];
+                if (consumer->type == tFullyConnected) ((dR_FC_Data*)consumer->layer)->drDeferredInput = n;
+                else ((dR_Softmax_Data*)consumer->layer)->drDeferredInput = n;
+                ((dR_Conv2d_Data*)c->layer)->drFusedAvgPool = TRUE;
+                ((dR_Pooling_Data*)n->layer)->drFused = TRUE;
+            }
         }
         if (n->type != tConcat) continue;
         dR_Concat_Data* cd = (dR_Concat_Data*)n->layer;

@@ -46,6 +46,9 @@ struct dR_Conv2d_Data {
     dR_Node*            drAbsorbed1x1;  /* set by the buffer planner on a Winograd node: the 1x1 sibling (same input, the channels
                                            just below this node's in a fused concat) whose filters ride along as centre taps */
     dR_Node*            drAbsorbedBy;   /* set on that 1x1 sibling: its compute() launches nothing */
+    gboolean            drFusedAvgPool; /* set by the buffer planner: a 1x1 layer whose only consumer is a global average
+                                           pooling read by an FC or softmax node; the layer leaves per-tile pixel sums
+                                           in workspaceBuf and neither its tensor nor the pooled one is computed by a kernel of its own */
     gboolean            drFusedPool;    /* set by the buffer planner: the node's only consumer is a 2x2/2 max pool and
                                            this node writes the pooled tensor straight into that node's buffer */
 };

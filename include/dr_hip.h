@@ -137,6 +137,14 @@ size_t drhip_conv3x3_winograd_workspace_floats(int W, int H, int I, int O, int v
  * [I][O]->[O][I] re-layout (Kernels/dR_conv2d1x1.cl:4-53, src/dR_nodes_conv2d.c:1605-1716). */
 int drhip_conv1x1_f32(const float* in, const float* w, const float* bias, float* out,
                       int P, int I, int O, int relu, int variant, void* stream);
+/* 1x1 convolution followed by a global average pooling, without the [O][P] tensor in between:
+ * partials[t*O + o] = sum over the pixels p of pixel tile t (32 pixels each) of act(b[o] + w . in[.][p]).
+ * The pooled value of channel o is (sum_t partials[t*O + o]) / P: hand the partials to the consumer
+ * as a drhip_deferred_vec {partials, NULL, drhip_conv1x1_poolsum_slices(P), O, 0, finished, P}.
+ * No counterpart in the reference, which runs conv2d1x1 and the pooling kernel one after the other. */
+int drhip_conv1x1_poolsum_slices(int P);
+int drhip_conv1x1_poolsum_f32(const float* in, const float* w, const float* bias, float* partials,
+                              int P, int I, int O, int relu, void* stream);
 /* Tile configuration for a 1x1 layer (replaces dR_conv2d_1x1_schedule, :1526-1602): waves per
  * output tile (1, 2, 4, 8 for 32x32 tiles; | 0x100 = 16x16 tiles, 1..16 waves, for small layers).
  * variant 0 in drhip_conv1x1_f32 = let the launcher pick. */
@@ -180,6 +188,8 @@ typedef struct drhip_deferred_vec {
     int slices, n, relu;
     float* finished;         /* NULL, or [n]: the consumer also stores the finished vector here (for a
                                 producer whose own output the caller wants to read) */
+    float divisor;           /* 0, or the finished element is divided by this last (sums of a global
+                                average pooling that its producer left as per-tile partial sums) */
 } drhip_deferred_vec;
 int drhip_fc_slices(int K, int N);
 int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, const float* Wt, const float* bias, float* y,

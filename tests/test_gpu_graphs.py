@@ -182,6 +182,41 @@ def test_fc_chain_fused(oracle, gpu):
         assert rel_err(outs[k], want[k + 1]) <= LAYER_TOL
 
 
+def test_conv_global_average_softmax_fused(oracle, gpu):
+    """1x1 conv -> global average pooling -> softmax (SqueezeNet's tail): the pooling kernel and the
+    convolution's tensor disappear; the pooled tensor, an output here, is stored by the softmax."""
+    rng = np.random.default_rng(9)
+    for tail in ("softmax", "fc"):
+        spec = [{"op": "feed", "shape": (13, 11, 24)},
+                {"op": "conv", "in": 0, "w": (rng.standard_normal((24, 70, 1, 1)) * 0.3).astype(np.float32), "b": (rng.standard_normal(70) * 0.05).astype(np.float32), "stride": (1, 1), "relu": True},
+                {"op": "pool", "in": 1, "window": (13, 11, 1), "stride": (13, 11, 1), "kind": 1}]
+        if tail == "softmax":
+            spec.append({"op": "softmax", "in": 2})
+        else:
+            spec.append({"op": "fc", "in": 2, "w": (rng.standard_normal((70, 300)) * 0.2).astype(np.float32), "b": (rng.standard_normal(300) * 0.05).astype(np.float32), "relu": False})
+        x = rng.random((24, 11, 13), dtype=np.float32)
+        want = oracle.run_spec(spec, {0: x})
+        res, launches = {}, {}
+        for mode in ("1", "0"):
+            os.environ["DR_FUSE_AVGPOOL"] = mode
+            try:
+                with dr.Environment() as env:
+                    g = env.create_graph()
+                    nodes = configs.build_graph(g, spec, [2, 3])
+                    dr.prepare(g)
+                    configs.feed_chw(nodes[0], x)
+                    assert g.lib.dR_apply(g.ptr) and g.lib.dR_apply(g.ptr)
+                    res[mode] = [a.copy() for a in configs.fetch_chw(g)]
+                    dr.graph_config(g).profilingGPU = 1
+                    assert g.lib.dR_apply(g.ptr)
+                    launches[mode] = g.lib.drhip_timing_count()
+            finally:
+                os.environ.pop("DR_FUSE_AVGPOOL", None)
+        assert launches["0"] - launches["1"] == 1, launches
+        for k in range(2):
+            assert rel_err(res["1"][k], want[2 + k]) <= LAYER_TOL and rel_err(res["1"][k], res["0"][k]) <= 1e-5
+
+
 def test_squeezenet_with_normalization_node(oracle, gpu):
     """Config 4 with its per-image normalisation moved into the graph: raw U[0,255) image in, a
     Normalization node (mean 0, deviation 1) in front of conv1."""
@@ -205,8 +240,9 @@ def test_config4_squeezenet(oracle, gpu):
     assert np.abs(logits - wl).max() <= LOGIT_TOL
     assert int(logits.argmax()) == int(wl.argmax()) and int(probs.argmax()) == int(want[-1].argmax())
     assert abs(float(probs.sum()) - 1) < 1e-4
-    # fused-concat production run gives the same final numbers as the all-outputs run
-    _, _, prod = run_config("squeezenet", env_vars={"DR_FUSE_EXPAND": "0"})
+    # fused-concat production run gives the same final numbers as the all-outputs run (the two fusions
+    # that change a summation order switched off)
+    _, _, prod = run_config("squeezenet", env_vars={"DR_FUSE_EXPAND": "0", "DR_FUSE_AVGPOOL": "0"})
     assert np.array_equal(prod[len(spec) - 1], got[len(spec) - 1])
     # and with the expand pairs of the 8 fire modules fused into single Winograd launches
     _, _, fused = run_config("squeezenet")

@@ -248,7 +248,8 @@ def test_fc(lib, dev, oracle, C, H, W, N, relu):
 
 class DeferredVec(ctypes.Structure):
     """drhip_deferred_vec (include/dr_hip.h)."""
-    _fields_ = [("partials", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("slices", ctypes.c_int), ("n", ctypes.c_int), ("relu", ctypes.c_int), ("finished", ctypes.c_void_p)]
+    _fields_ = [("partials", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("slices", ctypes.c_int), ("n", ctypes.c_int), ("relu", ctypes.c_int), ("finished", ctypes.c_void_p),
+                ("divisor", ctypes.c_float)]
 
 
 @pytest.mark.parametrize("N2", [1000, 2500])        # softmax with the vector in registers / re-read from memory
@@ -294,6 +295,26 @@ def test_fc_chain_without_finishing_kernels(lib, dev, oracle, N2):
     bad = DeferredVec(q1.value, b1d.value, s1, N1 + 1, 1, None)
     assert lib.drhip_fc_ex_f32(None, ctypes.byref(bad), W2d, b2d, y2b, q2, N1, N2, 0, 0, None) == -1
     assert lib.drhip_fc_ex_f32(xd, None, W1d, b1d, None, None, 64, 8, 0, 1, None) == -1        # unsplit layers cannot defer
+
+
+@pytest.mark.parametrize("P,I,O,relu", [(196, 512, 1000, 1), (196, 64, 40, 0), (33, 9, 65, 1), (1, 1, 1, 0), (70, 24, 31, 1)])
+def test_conv1x1_with_global_average(lib, dev, oracle, P, I, O, relu):
+    """1x1 convolution whose epilogue leaves per-tile pixel sums; the softmax in front of which the
+    pooled vector is needed adds the tiles and divides (drhip_deferred_vec.divisor)."""
+    x, w, b = rnd(I, 1, P), rnd(I, O, 1, 1, scale=np.sqrt(2.0 / I)), rnd(O, scale=0.05)
+    conv = oracle.conv1x1(x, w, b, relu=bool(relu))                      # [O, 1, P]
+    pooled = oracle.pool(conv, (P, 1, 1), (P, 1, 1), 1).reshape(-1)       # global average
+    slices = lib.drhip_conv1x1_poolsum_slices(P)
+    assert slices == (P + 31) // 32
+    parts = dev.empty(slices * O)
+    ok(lib, lib.drhip_conv1x1_poolsum_f32(dev.put(x), dev.put(w), dev.put(b), parts, P, I, O, relu, None))
+    got = dev.get(parts, (slices, O)).astype(np.float64).sum(axis=0) / P
+    assert rel_err(got, pooled) <= TOL
+    fin, prob = dev.empty(O), dev.empty(O)
+    d = DeferredVec(parts.value, None, slices, O, 0, fin.value, float(P))
+    ok(lib, lib.drhip_softmax_ex_f32(None, ctypes.byref(d), prob, O, None))
+    assert rel_err(dev.get(fin, (O,)), pooled) <= TOL
+    assert rel_err(dev.get(prob, (O,)), oracle.softmax(pooled)) <= TOL
 
 
 @pytest.mark.parametrize("C,H,W", [(3, 224, 224), (1, 5, 7), (4, 17, 33), (64, 56, 56), (1, 1, 2)])
