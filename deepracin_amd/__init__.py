@@ -163,6 +163,9 @@ def load_library(path=None):
         "drhip_timing_count": (c_int, []),
         "drhip_timing_end": (c_int, [POINTER(c_float), c_int, POINTER(c_int)]),
         "drhip_conv2d_direct_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 9 + [vp]),
+        "drhip_conv3x3_pool3s2_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 7 + [vp]),
+        "drhip_conv1x1_poolsum_f32": (c_int, [vp, vp, vp, vp, c_int, c_int, c_int, c_int, vp]),
+        "drhip_conv1x1_poolsum_slices": (c_int, [c_int]),
         "drhip_winograd_filter_transform_f32": (c_int, [vp, vp, c_int, c_int, vp]),
         "drhip_conv3x3_winograd_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 6 + [vp, vp]),
         "drhip_conv3x3_winograd_filter_floats": (c_size_t, [c_int, c_int]),

@@ -16,6 +16,8 @@
 // broadcast reads), then every lane runs kw*kh*OCT FMAs per channel out of LDS.
 #include "drhip_common.hpp"
 
+#include <cfloat>
+
 namespace drhip {
 
 constexpr int kDirTile = 16;            // output tile edge
@@ -157,6 +159,120 @@ conv_direct_fewc_kernel(const float* __restrict__ in, const float* __restrict__ 
     }
 }
 
+
+// First layer and the 3x3 / stride-2 max pooling behind it in one kernel, on the matrix cores.
+//
+// A workgroup owns a 4x4 tile of POOLED pixels x 16*MB channels.  The pooling windows of that tile
+// cover 9x9 convolution outputs (81, dealt to six wavefronts as six 16-pixel MFMA columns); each
+// wavefront computes its 16 pixels for all channels as a small GEMM over k = (channel, tap), 9*I <= 36
+// values = up to 9 k-steps of v_mfma_f32_16x16x4_f32 (B: gathered input samples, zero padding by
+// select; A: the filters [I][O][9] as they are), adds bias, applies ReLU, and parks the pixels in
+// LDS; then all lanes pool out of LDS in the pooling kernel's scan order.  Convolution outputs
+// outside the map count as 0.0, exactly what the pooling kernel reads there.  The full-resolution
+// tensor (3.2 MB for SqueezeNet's conv1) is never written; the halo costs (9/8)^2 = 1.27x the MFMAs.
+constexpr int kFpPool = 4;                          // pooled tile edge
+constexpr int kFpConv = 2 * kFpPool + 1;            // convolution tile edge
+constexpr int kFpPix = kFpConv * kFpConv;           // 81
+constexpr int kFpWaves = (kFpPix + 15) / 16;        // 6
+constexpr int kFpThreads = 64 * kFpWaves;
+constexpr int kFpPitch = 16 * kFpWaves + 1;         // LDS row pitch (floats)
+typedef float f32x4d __attribute__((ext_vector_type(4)));
+
+template <int MB, int KS>                           // KS = k-steps = ceil(9*I / 4)
+__global__ void __launch_bounds__(kFpThreads)
+conv3x3_fewc_pool3s2_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
+                            float* __restrict__ out, int W, int H, int I, int O, int Wo, int Ho, int Wp, int Hp,
+                            int sx, int sy, int tilesX, int relu) {
+    __shared__ float convT[16 * MB * kFpPitch];
+    __shared__ float wT[4 * KS * 16 * MB];          // filters as [k = (channel, tap)][channel out], zero padded
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15, lk = lane >> 4;
+    const int tileX = blockIdx.x % tilesX, tileY = blockIdx.x / tilesX;
+    const int o0 = blockIdx.y * 16 * MB;
+
+    const int q = 16 * wave + j;                    // convolution pixel within the 9x9 tile
+    const int ry = q / kFpConv, rx = q % kFpConv;
+    const int cy = 2 * kFpPool * tileY + ry, cx = 2 * kFpPool * tileX + rx;
+    const bool pixOk = q < kFpPix && cy < Ho && cx < Wo;
+
+    // B operands: this lane's input samples, gathered now ...
+    float b[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int kidx = 4 * ks + lk;               // (channel, tap)
+        const int c = kidx / 9, tap = kidx % 9;
+        const int iy = cy * sy + tap / 3 - 1, ix = cx * sx + tap % 3 - 1;
+        const bool ok = pixOk && kidx < 9 * I && iy >= 0 && iy < H && ix >= 0 && ix < W;
+        const float v = in[((size_t)min(c, I - 1) * H + min(max(iy, 0), H - 1)) * W + min(max(ix, 0), W - 1)];
+        b[ks] = ok ? v : 0.0f;
+    }
+    // ... while the workgroup's filters go to LDS once, read in their own order (contiguous per
+    // input channel: w[c][o0 ..][9]) and written transposed, so that an MFMA A operand is 16
+    // consecutive floats.
+    constexpr int OBc = 16 * MB;
+    constexpr int kRounds = (4 * KS * OBc + kFpThreads - 1) / kFpThreads;
+    float fv[kRounds];
+    int dst[kRounds];
+#pragma unroll
+    for (int u = 0; u < kRounds; ++u) {             // all loads first (clamped addresses), one trip to memory
+        const int e = tid + u * kFpThreads;
+        // e -> (c, o local, tap) in memory order for real filter values, the zero padding after them
+        const bool real = e < 9 * I * OBc;
+        const int c = min(e / (9 * OBc), I - 1), rest = e % (9 * OBc);
+        const int ol = real ? rest / 9 : (e - 9 * I * OBc) % OBc;
+        const int kidx = real ? c * 9 + rest % 9 : 9 * I + (e - 9 * I * OBc) / OBc;
+        const float f = w[((size_t)c * O + min(o0 + ol, O - 1)) * 9 + rest % 9];
+        fv[u] = (real && o0 + ol < O) ? f : 0.0f;
+        dst[u] = e < 4 * KS * OBc ? kidx * OBc + ol : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kRounds; ++u)
+        if (dst[u] >= 0) wT[dst[u]] = fv[u];
+    __syncthreads();
+    float a[MB][KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) a[m][ks] = wT[(4 * ks + lk) * OBc + 16 * m + j];
+    f32x4d acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = f32x4d{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int m = 0; m < MB; ++m) acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[m][ks], b[ks], acc[m], 0, 0, 0);
+
+    // D: lane -> pixel j, register r -> channel 4*lk + r of block m
+#pragma unroll
+    for (int m = 0; m < MB; ++m)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int ch = 16 * m + 4 * lk + r;
+            float v = acc[m][r] + ((bias && o0 + ch < O) ? bias[o0 + ch] : 0.0f);
+            if (relu) v = fmaxf(v, 0.0f);
+            convT[ch * kFpPitch + q] = pixOk ? v : 0.0f;
+        }
+    __syncthreads();
+
+    for (int idx = tid; idx < 16 * MB * kFpPool * kFpPool; idx += kFpThreads) {
+        const int ch = idx / (kFpPool * kFpPool), pp = idx % (kFpPool * kFpPool);
+        const int ppy = pp / kFpPool, ppx = pp % kFpPool;
+        const int py = kFpPool * tileY + ppy, px = kFpPool * tileX + ppx;
+        if (py < Hp && px < Wp && o0 + ch < O) {
+            float r = -FLT_MAX;
+#pragma unroll
+            for (int dy = 0; dy < 3; ++dy)
+#pragma unroll
+                for (int dx = 0; dx < 3; ++dx) {
+                    const float v = convT[ch * kFpPitch + (2 * ppy + dy) * kFpConv + 2 * ppx + dx];
+                    if (v > r) r = v;
+                }
+            out[((size_t)(o0 + ch) * Hp + py) * Wp + px] = r;
+        }
+    }
+}
+
 template <int OCT>
 static int launch_direct(const float* in, const float* w, const float* bias, float* out,
                          int W, int H, int I, int O, int kw, int kh, int sx, int sy, int relu, hipStream_t s) {
@@ -212,4 +328,24 @@ extern "C" int drhip_conv2d_direct_f32(const float* in, const float* w, const fl
     if (O >= 8 && tiles * ceil_div(O, 8) >= num_cu())
         return launch_direct<8>(in, w, bias, out, W, H, I, O, kw, kh, strideX, strideY, relu, s);
     return launch_direct<4>(in, w, bias, out, W, H, I, O, kw, kh, strideX, strideY, relu, s);
+}
+
+extern "C" int drhip_conv3x3_pool3s2_f32(const float* in, const float* w, const float* bias, float* out,
+                                         int W, int H, int I, int O, int strideX, int strideY, int relu, void* stream) {
+    DRHIP_REQUIRE(in && w && out, "drhip_conv3x3_pool3s2_f32: NULL tensor");
+    DRHIP_REQUIRE(W > 0 && H > 0 && O > 0 && I >= 1 && I <= 4, "drhip_conv3x3_pool3s2_f32: bad shape %dx%dx%d -> %d (1 to 4 input channels)", W, H, I, O);
+    DRHIP_REQUIRE(strideX > 0 && strideY > 0 && W / strideX > 0 && H / strideY > 0, "drhip_conv3x3_pool3s2_f32: bad stride or empty output");
+    DRHIP_REQUIRE((long long)W * H * I < (1ll << 31) && (long long)W * H * O < (1ll << 31), "drhip_conv3x3_pool3s2_f32: tensor too large");
+    const int Wo = W / strideX, Ho = H / strideY, Wp = ceil_div(Wo, 2), Hp = ceil_div(Ho, 2);
+    const int tilesX = ceil_div(Wp, kFpPool), tilesY = ceil_div(Hp, kFpPool);
+    hipStream_t s = as_stream(stream);
+    const int ks = ceil_div(9 * I, 4);              // 3, 5, 7 or 9
+    const bool wide = O > 32;                       // 64 channels per workgroup, else 32
+    const dim3 grid(tilesX * tilesY, ceil_div(O, wide ? 64 : 32)), block(kFpThreads);
+#define DRHIP_FP(MBV, KSV) launch((conv3x3_fewc_pool3s2_kernel<MBV, KSV>), grid, block, 0, s, in, w, bias, out, W, H, I, O, Wo, Ho, Wp, Hp, strideX, strideY, tilesX, relu)
+#define DRHIP_FP_K(MBV) do { if (ks == 3) DRHIP_FP(MBV, 3); else if (ks == 5) DRHIP_FP(MBV, 5); else if (ks == 7) DRHIP_FP(MBV, 7); else DRHIP_FP(MBV, 9); } while (0)
+    if (wide) DRHIP_FP_K(4); else DRHIP_FP_K(2);
+#undef DRHIP_FP_K
+#undef DRHIP_FP
+    return launched("conv3x3_fewc_pool3s2_kernel");
 }

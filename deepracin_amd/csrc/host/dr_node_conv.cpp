@@ -187,8 +187,11 @@ gboolean conv_compute(dR_Graph* net, dR_Node* node) {
                 rc = drhip_conv1x1_f32(in, w, b, out, W * H, I, O, relu, c->variant, stream_of(net));
             break;
         default:
-            rc = drhip_conv2d_direct_f32(in, w, b, out, W, H, I, O, c->shape.s0, c->shape.s1,
-                                         c->stride.s1, c->stride.s2, relu, stream_of(net));
+            if (c->drFusedPool)                 // first layer + the 3x3/2 max pool behind it (out = the pool's buffer)
+                rc = drhip_conv3x3_pool3s2_f32(in, w, b, out, W, H, I, O, c->stride.s1, c->stride.s2, relu, stream_of(net));
+            else
+                rc = drhip_conv2d_direct_f32(in, w, b, out, W, H, I, O, c->shape.s0, c->shape.s1,
+                                             c->stride.s1, c->stride.s2, relu, stream_of(net));
             break;
     }
     return !device_failed(net, rc, "deepRACIN:conv2d");

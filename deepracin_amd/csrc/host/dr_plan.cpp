@@ -67,22 +67,31 @@ bool expand_pair(const dR_Node* a, const dR_Node* b) {
     return ia.size() == 1 && ib.size() == 1 && ia[0] == ib[0];
 }
 
-// A 2x2 / stride-2 max pool directly behind a Winograd convolution: every 2x2 output tile of the
-// convolution is one pooling window, so the convolution's epilogue can store the maximum and the
-// full-resolution tensor never exists.  Only when nobody else wants that tensor.
+// Max pooling stored by the convolution in front of it, so that the full-resolution tensor never
+// exists (only when nobody else wants that tensor; DR_FUSE_POOL=0 keeps the two apart):
+//  - a 2x2 / stride-2 pool behind a Winograd convolution: every 2x2 output tile of the convolution
+//    is one pooling window;
+//  - a 3x3 / stride-2 pool behind a first layer (3x3 filter, at most 4 input channels): one kernel
+//    computes the convolution outputs of a pooled tile on the matrix cores and pools them in LDS.
 dR_Node* pool_fusable_producer(const dR_Node* p) {
     if (p->type != tPooling) return nullptr;
     const char* env = getenv("DR_FUSE_POOL");
     if (env && strcmp(env, "0") == 0) return nullptr;
     const dR_Pooling_Data* pd = (const dR_Pooling_Data*)p->layer;
-    if (pd->poolingType != tMax || pd->shape.s1 != 2 || pd->shape.s2 != 2 || pd->shape.s3 != 1 ||
-        pd->stride.s1 != 2 || pd->stride.s2 != 2 || pd->stride.s3 != 1) return nullptr;
+    if (pd->poolingType != tMax || pd->shape.s3 != 1 || pd->stride.s1 != 2 || pd->stride.s2 != 2 || pd->stride.s3 != 1) return nullptr;
+    const bool two = pd->shape.s1 == 2 && pd->shape.s2 == 2, three = pd->shape.s1 == 3 && pd->shape.s2 == 3;
+    if (!two && !three) return nullptr;
     std::vector<dR_Node*> ins = nodes_of(p->previous_layers);
     if (ins.size() != 1) return nullptr;
     dR_Node* c = ins[0];
-    if (c->type != tConv2d || ((const dR_Conv2d_Data*)c->layer)->algo != drConvWinograd) return nullptr;
+    if (c->type != tConv2d) return nullptr;
+    const dR_Conv2d_Data* cd = (const dR_Conv2d_Data*)c->layer;
     if (c->output || c->outputBuf || !c->next_layers || c->next_layers->length != 1) return nullptr;
-    if ((c->oshape.s0 | c->oshape.s1) & 1) return nullptr;
+    if (two) {
+        if (cd->algo != drConvWinograd || ((c->oshape.s0 | c->oshape.s1) & 1)) return nullptr;
+    } else {
+        if (cd->algo != drConvDirect || cd->shape.s0 != 3 || cd->shape.s1 != 3 || cd->shape.s2 > 4) return nullptr;
+    }
     return c;
 }
 

@@ -99,6 +99,14 @@ int drhip_conv2d_direct_f32(const float* in, const float* w, const float* bias, 
                             int W, int H, int I, int O, int kw, int kh,
                             int strideX, int strideY, int relu, void* stream);
 
+/* First layer (1 to 4 input channels, 3x3, any stride, zero padding, bias, optional ReLU) followed by
+ * a 3x3 / stride-2 max pooling with the reference's pooling rules (out = ceil(in/2), samples outside
+ * the map read 0.0): out[O][ceil(Ho/2)][ceil(Wo/2)], Wo = W/strideX, Ho = H/strideY.  The
+ * convolution's own tensor is never written.  Replaces the generated conv kernel plus the generated
+ * pooling kernel of such a pair (src/dR_nodes_conv2d.c:481-773, src/dR_nodes_pooling.c:277-401). */
+int drhip_conv3x3_pool3s2_f32(const float* in, const float* w, const float* bias, float* out,
+                              int W, int H, int I, int O, int strideX, int strideY, int relu, void* stream);
+
 /* Winograd F(2x2,3x3) filter transform U = G g G^T for every (c,o).  Runs once per layer at
  * dR_prepare time.  U holds drhip_conv3x3_winograd_filter_floats(I,O) floats in the layout the MFMA
  * kernel streams: U[xi][c/8][o][8] with xi = 4*row+col, input channels padded with zeros to a

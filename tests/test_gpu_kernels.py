@@ -83,6 +83,27 @@ def test_conv_direct(lib, dev, oracle, W, H, I, O, k, s):
     assert rel_err(dev.get(out, want2.shape), want2) <= TOL
 
 
+@pytest.mark.parametrize("W,H,I,O,sx,sy", [(224, 224, 3, 64, 2, 2), (33, 31, 3, 9, 2, 2), (17, 13, 1, 5, 1, 1), (20, 18, 4, 70, 1, 2),
+                                            (8, 5, 2, 16, 3, 1), (2, 2, 3, 2, 1, 1), (9, 9, 4, 33, 2, 2), (64, 48, 3, 32, 1, 1)])
+@pytest.mark.parametrize("relu", [1, 0])
+def test_first_layer_conv_with_maxpool(lib, dev, oracle, W, H, I, O, sx, sy, relu):
+    """3x3 first-layer convolution + 3x3/2 max pooling in one kernel against the two oracle steps.
+    Without ReLU the convolution has negative outputs, so the pooling's zero padding is visible."""
+    x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.05)
+    conv = oracle.conv_direct(x, w, b, (sx, sy), relu=bool(relu))
+    want = oracle.pool(conv, (3, 3, 1), (2, 2, 1), 0)
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_conv3x3_pool3s2_f32(dev.put(x), dev.put(w), dev.put(b), out, W, H, I, O, sx, sy, relu, None))
+    got = dev.get(out, want.shape)
+    assert rel_err(got, want) <= TOL
+    assert rel_err(got, oracle.pool_f64(oracle.conv_f64(x, w, b, stride=(sx, sy), relu=bool(relu)), (3, 3, 1), (2, 2, 1), 0)) <= TOL
+    # no bias
+    want2 = oracle.pool(oracle.conv_direct(x, w, None, (sx, sy), relu=bool(relu)), (3, 3, 1), (2, 2, 1), 0)
+    ok(lib, lib.drhip_conv3x3_pool3s2_f32(dev.put(x), dev.put(w), None, out, W, H, I, O, sx, sy, relu, None))
+    assert rel_err(dev.get(out, want2.shape), want2) <= TOL
+    assert lib.drhip_conv3x3_pool3s2_f32(dev.put(x), dev.put(w), None, out, W, H, 5, O, sx, sy, relu, None) == -1
+
+
 def wino_filters(lib, dev, w):
     I, O = w.shape[:2]
     n = lib.drhip_conv3x3_winograd_filter_floats(I, O)

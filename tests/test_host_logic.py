@@ -299,12 +299,15 @@ def test_schedule_order_and_buffer_plan(lib, oracle, name):
         for j in ins:
             last_use[j] = max(last_use[j], pos[i])
     fused_into = {}
-    # a 2x2/2 max pool behind a Winograd convolution is stored by the convolution itself: the
-    # convolution then owns no tensor of its own, only the pooled one in the pooling node's buffer
+    # a max pool stored by the convolution in front of it: the convolution then owns no tensor of
+    # its own, only the pooled one in the pooling node's buffer
     for i, n in enumerate(spec):
         if n["op"] == "pool" and plan[n["in"]][0] == plan[i][0]:
             j = n["in"]
-            assert spec[j]["op"] == "conv" and tuple(n["window"]) == (2, 2, 1) and tuple(n["stride"]) == (2, 2, 1) and n["kind"] == 0
+            # 2x2/2 behind a Winograd convolution, or 3x3/2 behind a first layer (3x3 filter, <= 4 input channels)
+            assert spec[j]["op"] == "conv" and tuple(n["stride"]) == (2, 2, 1) and n["kind"] == 0
+            k = spec[j]["w"].shape
+            assert tuple(n["window"]) == (2, 2, 1) or (tuple(n["window"]) == (3, 3, 1) and k[0] <= 4 and tuple(k[2:]) == (3, 3))
             assert plan[j][1] == plan[i][1] == 0 and j not in outs
             assert sum(1 for k in inputs if j in inputs[k]) == 1
             fused_into[j] = i
