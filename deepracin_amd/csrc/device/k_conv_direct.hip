@@ -185,6 +185,7 @@ conv3x3_fewc_pool3s2_kernel(const float* __restrict__ in, const float* __restric
                             int sx, int sy, int tilesX, int relu) {
     __shared__ float convT[16 * MB * kFpPitch];
     __shared__ float wT[4 * KS * 16 * MB];          // filters as [k = (channel, tap)][channel out], zero padded
+    __shared__ float biasT[16 * MB];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 15, lk = lane >> 4;
@@ -226,9 +227,12 @@ conv3x3_fewc_pool3s2_kernel(const float* __restrict__ in, const float* __restric
         fv[u] = (real && o0 + ol < O) ? f : 0.0f;
         dst[u] = e < 4 * KS * OBc ? kidx * OBc + ol : -1;
     }
+    float bv = 0.0f;                                // the bias comes along in the same trip
+    if (tid < OBc && bias) bv = bias[min(o0 + tid, O - 1)];
 #pragma unroll
     for (int u = 0; u < kRounds; ++u)
         if (dst[u] >= 0) wT[dst[u]] = fv[u];
+    if (tid < OBc) biasT[tid] = bv;
     __syncthreads();
     float a[MB][KS];
 #pragma unroll
@@ -249,7 +253,7 @@ conv3x3_fewc_pool3s2_kernel(const float* __restrict__ in, const float* __restric
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int ch = 16 * m + 4 * lk + r;
-            float v = acc[m][r] + ((bias && o0 + ch < O) ? bias[o0 + ch] : 0.0f);
+            float v = acc[m][r] + biasT[ch];
             if (relu) v = fmaxf(v, 0.0f);
             convT[ch * kFpPitch + q] = pixOk ? v : 0.0f;
         }
