@@ -42,8 +42,8 @@ PEAK_HBM_GBS = 8000.0
 # runs of this script, scaled by what the same counters read for a copy of known size; the
 # commands and the per-layer figures are in profiles/.  Keyed by (workload, kernel group).
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    ("vgg16", "winograd"): 24935.4 * 1024,      # profiles/vgg16_hbm_traffic.md: fetch 263 376 + write 60 784 KiB over 13 launches
-    ("vgg16", "fc"): 167697.6 * 1024,         # fetch 501 560 + write 1 533 KiB over 3 launches
+    ("vgg16", "winograd"): 24935.9 * 1024,      # profiles/vgg16_hbm_traffic.md: fetch 263 376 + write 60 784 KiB over 13 launches
+    ("vgg16", "fc"): 167699.2 * 1024,         # fetch 501 560 + write 1 533 KiB over 3 launches
 }
 
 
