@@ -277,6 +277,150 @@ conv3x3_fewc_pool3s2_kernel(const float* __restrict__ in, const float* __restric
     }
 }
 
+// Direct 3x3 convolution on the matrix cores (stride 1 or 2, more than 4 input channels): the
+// implicit GEMM  out[o][p] = sum_{c,tap} w[c][o][tap] * in[c][pixel p shifted by tap],  K = 9*I.
+//
+// A workgroup (4 waves) owns 32 output channels x NY MFMA column groups of 32 output pixels (a
+// 16 x 2*NY block; NY = 2 for layers large enough to fill the chip that way: a staged filter then
+// feeds two MFMAs) and walks the input channels 16 at a time.  A stage's zero-padded input patch and
+// its filters (re-laid [c][tap][o]) are staged in LDS by all lanes, double buffered: the global
+// loads of stage s+1 are in flight while stage s is multiplied.  Inside a stage the four waves
+// split the channels (4 each = two k-steps of v_mfma_f32_32x32x2_f32 per tap, 18 MFMAs), every
+// operand is one ds_read_b32; the four partial tiles meet in LDS at the end (wave order, so the
+// summation order is fixed), then bias, ReLU and 64-byte row stores.  Small layers get enough
+// workgroups from the small pixel block (56x56 -> 64 channels: 224), large ones are MFMA-bound.
+constexpr int kDmTX = 16;                   // output block: 16 x 2*NY pixels
+constexpr int kDmCC = 16;                   // input channels per stage
+constexpr int kDmThreads = 256;
+constexpr int kDmPartPitch = 33;
+
+template <int S, int NY>                    // stride (both directions): 1 or 2; column groups per wave
+__global__ void __launch_bounds__(kDmThreads)
+conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
+                           float* __restrict__ out, int W, int H, int I, int O, int Wo, int Ho, int tilesX, int relu) {
+    constexpr int kDmTY = 2 * NY;
+    constexpr int PH = (kDmTY - 1) * S + 3, PW = (kDmTX - 1) * S + 3;      // input patch of the block
+    constexpr int kPatch = kDmCC * PH * PW, kFilt = kDmCC * 9 * 32;         // floats per stage
+    constexpr int kPatchLoads = (kPatch + kDmThreads - 1) / kDmThreads;
+    constexpr int kFiltLoads = (kFilt / 4 + kDmThreads - 1) / kDmThreads;   // 16-byte loads
+    extern __shared__ float lds[];              // [2][kPatch + kFilt]; reused for the partial tiles at the end
+    typedef float f32x16d __attribute__((ext_vector_type(16)));
+    typedef float f32x4l __attribute__((ext_vector_type(4)));
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 31, kpar = lane >> 5;
+    const int xx = j & 15, yy = j >> 4;
+    const int tileX = blockIdx.x % tilesX, tileY = blockIdx.x / tilesX;
+    const int o0 = blockIdx.y * 32;
+    const int x0 = tileX * kDmTX, y0 = tileY * kDmTY;
+    const int ix0 = x0 * S - 1, iy0 = y0 * S - 1;
+    const int nStages = (I + kDmCC - 1) / kDmCC;
+    const bool wholeTile = o0 + 32 <= O;        // the 16-byte filter loads need all 32 channels to exist
+
+    float pv[kPatchLoads];
+    f32x4l fv[kFiltLoads];
+    auto load_stage = [&](int s) {
+        const int c0 = s * kDmCC;
+#pragma unroll
+        for (int u = 0; u < kPatchLoads; ++u) {
+            const int e = tid + u * kDmThreads;
+            const int c = min(e / (PH * PW), kDmCC - 1), rem = e % (PH * PW);
+            const int gy = iy0 + rem / PW, gx = ix0 + rem % PW;
+            const bool ok = e < kPatch && c0 + c < I && gy >= 0 && gy < H && gx >= 0 && gx < W;
+            const float v = in[((size_t)min(c0 + c, I - 1) * H + min(max(gy, 0), H - 1)) * W + min(max(gx, 0), W - 1)];
+            pv[u] = ok ? v : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < kFiltLoads; ++u) {
+            const int f = 4 * (tid + u * kDmThreads);                       // first of four floats in [c][o][tap] order
+            const int c = min(f / 288, kDmCC - 1), rem = f % 288;
+            if (wholeTile && c0 + kDmCC <= I) {                             // workgroup-uniform
+                fv[u] = *(const f32x4l*)(w + ((size_t)(c0 + c) * O + o0) * 9 + rem);
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int ol = (rem + k) / 9, tap = (rem + k) % 9;
+                    const float v = w[((size_t)min(c0 + c, I - 1) * O + min(o0 + ol, O - 1)) * 9 + tap];
+                    fv[u][k] = (c0 + c < I && o0 + ol < O) ? v : 0.0f;
+                }
+            }
+        }
+    };
+    auto store_stage = [&](float* buf) {
+        float* patch = buf;
+        float* filt = buf + kPatch;
+#pragma unroll
+        for (int u = 0; u < kPatchLoads; ++u) {
+            const int e = tid + u * kDmThreads;
+            if (e < kPatch) patch[e] = pv[u];
+        }
+#pragma unroll
+        for (int u = 0; u < kFiltLoads; ++u) {
+            const int f = 4 * (tid + u * kDmThreads);
+            if (f < kFilt) {
+                const int c = f / 288, rem = f % 288;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) filt[(c * 9 + (rem + k) % 9) * 32 + (rem + k) / 9] = fv[u][k];
+            }
+        }
+    };
+
+    f32x16d acc[NY];
+#pragma unroll
+    for (int g = 0; g < NY; ++g)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[g][r] = 0.0f;
+
+    load_stage(0);
+    store_stage(lds);
+    __syncthreads();
+    for (int s = 0; s < nStages; ++s) {
+        const float* buf = lds + (s & 1) * (kPatch + kFilt);
+        if (s + 1 < nStages) load_stage(s + 1);
+        const float* patch = buf;
+        const float* filt = buf + kPatch;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            const int ch = 4 * wave + 2 * ks + kpar;                        // channel within the stage
+#pragma unroll
+            for (int tap = 0; tap < 9; ++tap) {
+                const float a = filt[(ch * 9 + tap) * 32 + j];
+#pragma unroll
+                for (int g = 0; g < NY; ++g) {
+                    const float b = patch[(ch * PH + (2 * g + yy) * S + tap / 3) * PW + xx * S + tap % 3];
+                    acc[g] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[g], 0, 0, 0);
+                }
+            }
+        }
+        if (s + 1 < nStages) store_stage(lds + ((s + 1) & 1) * (kPatch + kFilt));
+        __syncthreads();
+    }
+
+    // partial tiles of the four waves -> LDS -> summed in wave order
+    float* part = lds;
+#pragma unroll
+    for (int g = 0; g < NY; ++g) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            part[(wave * 32 + 8 * (r / 4) + 4 * kpar + (r % 4)) * kDmPartPitch + j] = acc[g][r];
+        __syncthreads();
+        for (int idx = tid; idx < 32 * 32; idx += kDmThreads) {
+            const int ol = idx >> 5, pl = idx & 31;
+            const int o = o0 + ol, x = x0 + (pl & 15), y = y0 + 2 * g + (pl >> 4);
+            float v = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) v += part[(k * 32 + ol) * kDmPartPitch + pl];
+            if (o < O && x < Wo && y < Ho) {
+                if (bias) v += bias[o];
+                if (relu) v = fmaxf(v, 0.0f);
+                out[((size_t)o * Ho + y) * Wo + x] = v;
+            }
+        }
+        if (g + 1 < NY) __syncthreads();        // the partial tiles are overwritten by the next group
+    }
+}
+
 template <int OCT>
 static int launch_direct(const float* in, const float* w, const float* bias, float* out,
                          int W, int H, int I, int O, int kw, int kh, int sx, int sy, int relu, hipStream_t s) {
@@ -323,6 +467,24 @@ extern "C" int drhip_conv2d_direct_f32(const float* in, const float* w, const fl
 #undef DRHIP_FEWC_I
 #undef DRHIP_FEWC
         return launched("conv_direct_fewc_kernel");
+    }
+    if (kw == 3 && kh == 3 && strideX == strideY && (strideX == 1 || strideX == 2) && !getenv("DR_DIRECT_VALU")) {
+        // matrix-core form: 32 channels x (16 x 2) pixels per workgroup, 16 input channels per stage
+        const int Wo = W / strideX, Ho = H / strideY;
+        // 16 x 4 pixel blocks when those alone give every CU a workgroup, else 16 x 2 (stride 2
+        // always: its double-buffered patch of a 16 x 4 block would not fit 64 KiB of LDS)
+        const int ny = (strideX == 1 && ceil_div(Wo, kDmTX) * ceil_div(Ho, 4) * ceil_div(O, 32) >= num_cu()) ? 2 : 1;
+        const int tilesX = ceil_div(Wo, kDmTX), tilesY = ceil_div(Ho, 2 * ny);
+        const dim3 grid(tilesX * tilesY, ceil_div(O, 32)), block(kDmThreads);
+        const int PH = (2 * ny - 1) * strideX + 3, PW = (kDmTX - 1) * strideX + 3;
+        const size_t stage = (size_t)kDmCC * PH * PW + (size_t)kDmCC * 9 * 32;
+        const size_t ldsFloats = 2 * stage > (size_t)4 * 32 * kDmPartPitch ? 2 * stage : (size_t)4 * 32 * kDmPartPitch;
+        DRHIP_REQUIRE(ldsFloats * sizeof(float) <= 64 * 1024, "drhip_conv2d_direct_f32: internal: LDS stage too large");
+#define DRHIP_DM(SV, NYV) launch((conv3x3_direct_mfma_kernel<SV, NYV>), grid, block, ldsFloats * sizeof(float), s0, in, w, bias, out, W, H, I, O, Wo, Ho, tilesX, relu)
+        if (strideX == 1) { if (ny == 2) DRHIP_DM(1, 2); else DRHIP_DM(1, 1); }
+        else DRHIP_DM(2, 1);
+#undef DRHIP_DM
+        return launched("conv3x3_direct_mfma_kernel");
     }
     // Few output channels per lane when the tile count alone cannot fill the CUs.
     const int tiles = ceil_div(W / strideX, kDirTile) * ceil_div(H / strideY, kDirTile);

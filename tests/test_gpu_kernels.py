@@ -69,6 +69,7 @@ def ok(lib, rc):
     (224, 224, 3, 64, 3, 2),     # SqueezeNet conv1
     (17, 13, 5, 7, 3, 1), (20, 18, 4, 20, 5, 1), (33, 31, 3, 9, 3, 2), (16, 16, 2, 3, 7, 3), (9, 9, 1, 1, 1, 2),
     (37, 21, 4, 33, 3, 1), (8, 5, 1, 16, 3, 3), (2, 2, 3, 2, 3, 1),     # I <= 4 with a 3x3 filter: the no-LDS first-layer kernel
+    (112, 110, 24, 40, 3, 1), (61, 37, 17, 70, 3, 2), (30, 9, 8, 32, 3, 1),   # 3x3 on the matrix cores: 16x4 blocks, stride 2, ragged channels
 ])
 def test_conv_direct(lib, dev, oracle, W, H, I, O, k, s):
     x, w, b = np.abs(rnd(I, H, W)), rnd(I, O, k, k, scale=np.sqrt(2.0 / (k * k * I))), rnd(O, scale=0.01)
