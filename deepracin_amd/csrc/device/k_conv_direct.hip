@@ -17,6 +17,8 @@
 #include "drhip_common.hpp"
 
 #include <cfloat>
+#include <cstdlib>
+#include <cstring>
 
 namespace drhip {
 
@@ -468,7 +470,8 @@ extern "C" int drhip_conv2d_direct_f32(const float* in, const float* w, const fl
 #undef DRHIP_FEWC
         return launched("conv_direct_fewc_kernel");
     }
-    if (kw == 3 && kh == 3 && strideX == strideY && (strideX == 1 || strideX == 2) && !getenv("DR_DIRECT_VALU")) {
+    const char* valuOnly = getenv("DR_DIRECT_VALU");
+    if (kw == 3 && kh == 3 && strideX == strideY && (strideX == 1 || strideX == 2) && !(valuOnly && strcmp(valuOnly, "1") == 0)) {
         // matrix-core form: 32 channels x (16 x 2) pixels per workgroup, 16 input channels per stage
         const int Wo = W / strideX, Ho = H / strideY;
         // 16 x 4 pixel blocks when those alone give every CU a workgroup, else 16 x 2 (stride 2
