@@ -279,6 +279,84 @@ conv3x3_fewc_pool3s2_kernel(const float* __restrict__ in, const float* __restric
     }
 }
 
+// First layer without a pooling behind it (VGG16's conv1_1: 224x224x3 -> 64, stride 1): the same
+// small GEMM over k = (channel, tap) on v_mfma_f32_16x16x4_f32.  A workgroup of four waves owns a
+// 16 x 4 block of output pixels x 16*MB channels; a wave owns one row of 16 pixels (one MFMA column),
+// gathers its 9*I input samples (16 consecutive x per load), takes the filters from LDS (transposed
+// there once per workgroup) and stores 64-byte rows per channel.
+template <int MB, int KS>
+__global__ void __launch_bounds__(256)
+conv3x3_fewc_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
+                         float* __restrict__ out, int W, int H, int I, int O, int Wo, int Ho,
+                         int sx, int sy, int tilesX, int relu) {
+    constexpr int OBc = 16 * MB;
+    __shared__ float wT[4 * KS * OBc];              // filters as [k = (channel, tap)][channel out], zero padded
+    __shared__ float biasT[OBc];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15, lk = lane >> 4;
+    const int tileX = blockIdx.x % tilesX, tileY = blockIdx.x / tilesX;
+    const int o0 = blockIdx.y * OBc;
+    const int x = tileX * 16 + j, y = tileY * 4 + wave;
+    const bool pixOk = x < Wo && y < Ho;
+
+    float b[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+        const int kidx = 4 * ks + lk;               // (channel, tap)
+        const int c = kidx / 9, tap = kidx % 9;
+        const int iy = y * sy + tap / 3 - 1, ix = x * sx + tap % 3 - 1;
+        const bool ok = pixOk && kidx < 9 * I && iy >= 0 && iy < H && ix >= 0 && ix < W;
+        const float v = in[((size_t)min(c, I - 1) * H + min(max(iy, 0), H - 1)) * W + min(max(ix, 0), W - 1)];
+        b[ks] = ok ? v : 0.0f;
+    }
+    constexpr int kRounds = (4 * KS * OBc + 255) / 256;
+    float fv[kRounds];
+    int dst[kRounds];
+#pragma unroll
+    for (int u = 0; u < kRounds; ++u) {             // e -> (c, o local, tap) in memory order, then the zero padding
+        const int e = tid + u * 256;
+        const bool real = e < 9 * I * OBc;
+        const int c = min(e / (9 * OBc), I - 1), rest = e % (9 * OBc);
+        const int ol = real ? rest / 9 : (e - 9 * I * OBc) % OBc;
+        const int kidx = real ? c * 9 + rest % 9 : 9 * I + (e - 9 * I * OBc) / OBc;
+        const float f = w[((size_t)c * O + min(o0 + ol, O - 1)) * 9 + rest % 9];
+        fv[u] = (real && o0 + ol < O) ? f : 0.0f;
+        dst[u] = e < 4 * KS * OBc ? kidx * OBc + ol : -1;
+    }
+    float bv = 0.0f;
+    if (tid < OBc && bias) bv = bias[min(o0 + tid, O - 1)];
+#pragma unroll
+    for (int u = 0; u < kRounds; ++u)
+        if (dst[u] >= 0) wT[dst[u]] = fv[u];
+    if (tid < OBc) biasT[tid] = bv;
+    __syncthreads();
+
+    f32x4d acc[MB];
+#pragma unroll
+    for (int m = 0; m < MB; ++m) acc[m] = f32x4d{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+            acc[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(wT[(4 * ks + lk) * OBc + 16 * m + j], b[ks], acc[m], 0, 0, 0);
+
+    // D: lane -> pixel j, register r -> channel 4*lk + r of block m
+    if (pixOk) {
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int ch = 16 * m + 4 * lk + r;
+                if (o0 + ch < O) {
+                    float v = acc[m][r] + biasT[ch];
+                    if (relu) v = fmaxf(v, 0.0f);
+                    out[((size_t)(o0 + ch) * Ho + y) * Wo + x] = v;
+                }
+            }
+    }
+}
+
 // Direct 3x3 convolution on the matrix cores (stride 1 or 2, more than 4 input channels): the
 // implicit GEMM  out[o][p] = sum_{c,tap} w[c][o][tap] * in[c][pixel p shifted by tap],  K = 9*I.
 //
@@ -458,6 +536,22 @@ extern "C" int drhip_conv2d_direct_f32(const float* in, const float* w, const fl
     DRHIP_REQUIRE((long long)W * H * I < (1ll << 31) && (long long)(W / strideX) * (H / strideY) * O < (1ll << 31),
                   "drhip_conv2d_direct_f32: tensor too large");
     hipStream_t s0 = as_stream(stream);
+    const char* valuOnly = getenv("DR_DIRECT_VALU");
+    const bool valu = valuOnly && strcmp(valuOnly, "1") == 0;
+    if (I <= 4 && kw == 3 && kh == 3 && !valu) {
+        // first layers on the matrix cores: 16 x 4 pixels x 64 (32) channels per workgroup
+        const int Wo = W / strideX, Ho = H / strideY;
+        const int tilesX = ceil_div(Wo, 16), tilesY = ceil_div(Ho, 4);
+        const int ks = ceil_div(9 * I, 4);
+        const bool wide = O > 32;
+        const dim3 grid(tilesX * tilesY, ceil_div(O, wide ? 64 : 32)), block(256);
+#define DRHIP_FM(MBV, KSV) launch((conv3x3_fewc_mfma_kernel<MBV, KSV>), grid, block, 0, s0, in, w, bias, out, W, H, I, O, Wo, Ho, strideX, strideY, tilesX, relu)
+#define DRHIP_FM_K(MBV) do { if (ks == 3) DRHIP_FM(MBV, 3); else if (ks == 5) DRHIP_FM(MBV, 5); else if (ks == 7) DRHIP_FM(MBV, 7); else DRHIP_FM(MBV, 9); } while (0)
+        if (wide) DRHIP_FM_K(4); else DRHIP_FM_K(2);
+#undef DRHIP_FM_K
+#undef DRHIP_FM
+        return launched("conv3x3_fewc_mfma_kernel");
+    }
     if (I <= 4 && kw == 3 && kh == 3) {
         const int Wo = W / strideX, Ho = H / strideY;
         const int tilesX = ceil_div(Wo, kDirTile), tilesY = ceil_div(Ho, kDirTile);
@@ -470,8 +564,7 @@ extern "C" int drhip_conv2d_direct_f32(const float* in, const float* w, const fl
 #undef DRHIP_FEWC
         return launched("conv_direct_fewc_kernel");
     }
-    const char* valuOnly = getenv("DR_DIRECT_VALU");
-    if (kw == 3 && kh == 3 && strideX == strideY && (strideX == 1 || strideX == 2) && !(valuOnly && strcmp(valuOnly, "1") == 0)) {
+    if (kw == 3 && kh == 3 && strideX == strideY && (strideX == 1 || strideX == 2) && !valu) {
         // matrix-core form: 32 channels x (16 x 2) pixels per workgroup, 16 input channels per stage
         const int Wo = W / strideX, Ho = H / strideY;
         // 16 x 4 pixel blocks when those alone give every CU a workgroup, else 16 x 2 (stride 2

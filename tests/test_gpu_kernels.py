@@ -105,6 +105,21 @@ def test_first_layer_conv_with_maxpool(lib, dev, oracle, W, H, I, O, sx, sy, rel
     assert lib.drhip_conv3x3_pool3s2_f32(dev.put(x), dev.put(w), None, out, W, H, 5, O, sx, sy, relu, None) == -1
 
 
+def test_conv_direct_valu_kernels(lib, dev, oracle):
+    """DR_DIRECT_VALU=1: the LDS-tiled / first-layer VALU kernels behind the matrix-core forms."""
+    import os
+    os.environ["DR_DIRECT_VALU"] = "1"
+    try:
+        for (W, H, I, O, s) in [(56, 56, 64, 64, 1), (224, 224, 3, 64, 2), (33, 31, 3, 9, 2), (30, 9, 8, 32, 1)]:
+            x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
+            want = oracle.conv_direct(x, w, b, (s, s), relu=True)
+            out = dev.empty(want.size)
+            ok(lib, lib.drhip_conv2d_direct_f32(dev.put(x), dev.put(w), dev.put(b), out, W, H, I, O, 3, 3, s, s, 1, None))
+            assert rel_err(dev.get(out, want.shape), want) <= TOL
+    finally:
+        os.environ.pop("DR_DIRECT_VALU", None)
+
+
 def wino_filters(lib, dev, w):
     I, O = w.shape[:2]
     n = lib.drhip_conv3x3_winograd_filter_floats(I, O)
