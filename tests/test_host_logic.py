@@ -403,3 +403,13 @@ def test_pick_variants_are_launchable(lib):
         assert v >= 1
         c = lib.drhip_conv1x1_pick_variant(W * H, I, O)          # waves per tile | 0x100 for 16x16 tiles
         assert (c in (1, 2, 4, 8)) or (c & 0x100 and (c & 0xff) in (1, 2, 4, 8, 16) and c >> 9 == 0)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: any other --gpus value ends with a message, not with a number."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "exactly one GPU" in (r.stdout + r.stderr)
+    assert not r.stdout.strip().startswith("{")
