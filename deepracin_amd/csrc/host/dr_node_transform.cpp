@@ -368,4 +368,27 @@ dR_Node* dR_elemwise1op_parseAppendNode(dR_Graph* net, dR_Node** iNodes, gint nu
     return dR_ElemWise1Operation(net, iNodes[0], (dR_ElemWise1OperationType)op, (gfloat)atof(params[1]));
 }
 
+// ---- node types outside the CNN layer path -----------------------------------------------------------
+// The reference's ctypes wrapper resolves these names while it is imported
+// (python/deepracin/__init__.py.in:146-211); they keep the reference's signatures, append nothing and
+// return NULL, the way every constructor here reports a refused node.
+
+static dR_Node* outside_layer_path(const char* what) {
+    say("%s: node type outside the CNN layer path, not available in this build; no node appended.\n", what);
+    return NULL;
+}
+
+dR_Node* dR_MaskDependentFilter(dR_Graph*, dR_Node*, dR_Node*, dR_Shape3*) { return outside_layer_path("dR_MaskDependentFilter"); }
+void dR_MaskDependentFilter_setVariables(dR_Node*, gfloat*, gfloat*) { outside_layer_path("dR_MaskDependentFilter_setVariables"); }
+dR_Node* dR_PerPixelFilter(dR_Graph*, dR_Node*, dR_Node*, dR_Shape4*, dR_Shape4*) { return outside_layer_path("dR_PerPixelFilter"); }
+dR_Node* dR_ElemWise2Operation(dR_Graph*, dR_Node*, dR_Node*, dR_ElemWise2OperationType) { return outside_layer_path("dR_ElemWise2Operation"); }
+dR_Node* dR_ResolveRoI(dR_Graph*, dR_Node*, dR_Shape3*) { return outside_layer_path("dR_ResolveRoI"); }
+dR_Node* dR_RGB2gray(dR_Graph*, dR_Node*) { return outside_layer_path("dR_RGB2gray"); }
+dR_Node* dR_Upscaling(dR_Graph*, dR_Node*, dR_UpscalingType, gint, gint) { return outside_layer_path("dR_Upscaling"); }
+dR_Node* dR_LabelCreation(dR_Graph*, dR_Node*, dR_LabelCreationType, gfloat, gfloat, gfloat) { return outside_layer_path("dR_LabelCreation"); }
+dR_Node* dR_CropOrPad(dR_Graph*, dR_Node*, dR_Shape3*) { return outside_layer_path("dR_CropOrPad"); }
+// Called (not bound at import) by the wrapper's Conv2dTransposed(); unfinished in the reference itself.
+dR_Node* dR_Conv2dTransposed(dR_Graph*, dR_Node*, dR_Shape4, dR_Shape4, dR_ActivationType, gboolean) { return outside_layer_path("dR_Conv2dTransposed"); }
+void dR_Conv2dtransposed_setVariables(dR_Node*, gfloat*, gfloat*) { outside_layer_path("dR_Conv2dtransposed_setVariables"); }
+
 }  // extern "C"

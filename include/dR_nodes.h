@@ -188,6 +188,38 @@ struct dR_Normalization_Data {
 dR_Node* dR_Normalization(dR_Graph* net, dR_Node* inputLayer, dR_NormalizationType type, gfloat targetMean,
                           gfloat targetDev);
 
+/* ================================ nodes outside the CNN layer path ============================ */
+
+/* The reference's Python wrapper binds these constructors when it is imported
+ * (python/deepracin/__init__.py.in:146-211), so the symbols exist with the reference's signatures
+ * (include/dR_nodes_filter.h:61,63,161; dR_nodes_math.h:45; dR_nodes_misc.h:40,102,167,230;
+ * dR_nodes_transform.h:168).  The node types themselves (image filters, two-tensor arithmetic,
+ * region-of-interest, colour, upscaling, label and crop nodes) are not part of this build: every
+ * constructor prints which node type was asked for, appends nothing and returns NULL, and
+ * dR_MaskDependentFilter_setVariables does nothing. */
+enum dR_ElemWise2OperationType { tAdd, tSub, tMul, tDiv, tPow };
+typedef enum dR_ElemWise2OperationType dR_ElemWise2OperationType;
+enum dR_UpscalingType { tNearestNUp, tLinearUp, tBicubicUp };
+typedef enum dR_UpscalingType dR_UpscalingType;
+enum dR_LabelCreationType { t3to2ClassesBin, t3to2ClassesConf, t2ClassesBin, t2ClassesConf, tnClasses };
+typedef enum dR_LabelCreationType dR_LabelCreationType;
+
+dR_Node* dR_MaskDependentFilter(dR_Graph* net, dR_Node* inputImage, dR_Node* inputFilterMask, dR_Shape3* shape);
+void     dR_MaskDependentFilter_setVariables(dR_Node* layer, gfloat* weights, gfloat* bias);
+dR_Node* dR_PerPixelFilter(dR_Graph* net, dR_Node* inputImage, dR_Node* inputFilter, dR_Shape4* shape, dR_Shape4* stride);
+dR_Node* dR_ElemWise2Operation(dR_Graph* net, dR_Node* inputNode1, dR_Node* inputNode2, dR_ElemWise2OperationType op);
+dR_Node* dR_ResolveRoI(dR_Graph* net, dR_Node* inputLayer, dR_Shape3* shape);
+dR_Node* dR_RGB2gray(dR_Graph* net, dR_Node* inputLayer);
+dR_Node* dR_Upscaling(dR_Graph* net, dR_Node* inputLayer, dR_UpscalingType type, gint scaleFactorX, gint scaleFactorY);
+dR_Node* dR_LabelCreation(dR_Graph* net, dR_Node* inputLayer, dR_LabelCreationType type, gfloat class0offset,
+                          gfloat class1offset, gfloat class2offset);
+dR_Node* dR_CropOrPad(dR_Graph* net, dR_Node* inputLayer, dR_Shape3* targetshape);
+/* Looked up only when the wrapper's Conv2dTransposed() is called (include/dR_nodes_conv2d.h:229,245;
+ * shapes by value there); the node is unfinished in the reference. */
+dR_Node* dR_Conv2dTransposed(dR_Graph* net, dR_Node* inputnode, dR_Shape4 filtershape, dR_Shape4 stride,
+                             dR_ActivationType activation, gboolean useBias);
+void     dR_Conv2dtransposed_setVariables(dR_Node* node, gfloat* weights, gfloat* biases);
+
 #ifdef __cplusplus
 }
 #endif

@@ -41,6 +41,36 @@ def test_library_exports_every_declared_symbol(lib):
         assert must in syms
 
 
+def test_every_symbol_the_reference_python_wrapper_looks_up_resolves(lib):
+    """tests/golden/ref_wrapper_symbols.txt lists the lib.dR_* names of the reference's ctypes front-end
+    (python/deepracin/__init__.py.in:36-218 bind at import; a few more are looked up when called).  All
+    must resolve, or the unmodified wrapper stops with AttributeError before any graph is built."""
+    names = open(os.path.join(GOLDEN, "ref_wrapper_symbols.txt")).read().split()
+    assert len(names) >= 35 and "dR_MaskDependentFilter" in names and "dR_apply" in names
+    raw = ctypes.CDLL(dr.LIB_PATH)
+    missing = [s for s in names if not hasattr(raw, s)]
+    assert not missing, "looked up by the reference wrapper but not exported: %s" % missing
+
+
+def test_constructors_outside_the_layer_path_refuse(lib, capfd):
+    """Image-filter, two-tensor, RoI, colour, upscaling, label and crop constructors exist for the wrapper's
+    import only: they append nothing and return NULL."""
+    raw = ctypes.CDLL(dr.LIB_PATH)
+    g = lib.dR_NewGraph()
+    sh = (ctypes.c_int * 4)(3, 3, 1, 1)
+    for name, args in (("dR_RGB2gray", (g, None)), ("dR_ResolveRoI", (g, None, sh)), ("dR_CropOrPad", (g, None, sh)),
+                       ("dR_ElemWise2Operation", (g, None, None, 0)), ("dR_Upscaling", (g, None, 0, 2, 2)),
+                       ("dR_MaskDependentFilter", (g, None, None, sh)), ("dR_PerPixelFilter", (g, None, None, sh, sh)),
+                       ("dR_LabelCreation", (g, None, 0, ctypes.c_float(0), ctypes.c_float(0), ctypes.c_float(0)))):
+        f = getattr(raw, name)
+        f.restype = ctypes.c_void_p
+        assert f(*args) is None, name
+    raw.dR_MaskDependentFilter_setVariables.restype = None
+    raw.dR_MaskDependentFilter_setVariables(None, None, None)
+    out = capfd.readouterr().out
+    assert out.count("outside the CNN layer path") == 9
+
+
 def test_no_device_is_reported_not_faked(lib):
     # on a machine without a GPU the device layer says so; on a GPU box it initialises
     info = dr.DeviceInfo()
