@@ -176,6 +176,8 @@ def load_library(path=None):
         "drhip_pool_f32": (c_int, [vp, vp, vp] + [c_int] * 10 + [vp]),
         "drhip_fc_scratch_floats": (c_size_t, [c_int, c_int]),
         "drhip_fc_f32": (c_int, [vp] * 5 + [c_int] * 3 + [vp]),
+        "drhip_fc_noalloc_f32": (c_int, [vp] * 4 + [c_int] * 3 + [vp]),
+        "drhip_fc_noalloc_max_scratch_floats": (c_size_t, []),
         "drhip_fc_permute_rows_f32": (c_int, [vp, vp] + [c_int] * 4 + [vp]),
         "drhip_softmax_f32": (c_int, [vp, vp, c_int, vp]),
         "drhip_copy3d_f32": (c_int, [vp] + [c_int] * 5 + [vp] + [c_int] * 8 + [vp]),

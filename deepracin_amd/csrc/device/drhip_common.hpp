@@ -96,6 +96,9 @@ __device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {
 // Number of compute units of the active device (cached by drhip_init; 256 on MI355X).
 int num_cu();
 
+// Per-device set-up of the fully-connected kernels' built-in scratch (k_fc.hip); `device` must be current.
+int fc_static_scratch_setup(int device);
+
 }  // namespace drhip
 
 #define DRHIP_REQUIRE(cond, ...)                                   \

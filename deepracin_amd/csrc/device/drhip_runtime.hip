@@ -52,6 +52,7 @@ int drhip_init(int device, drhip_device_info* info) {
     if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
         return fail(DRHIP_ENODEVICE, "device %d is %s; this library carries gfx950 code only", device, p.gcnArchName);
     g_num_cu = p.multiProcessorCount;
+    if (int rc = fc_static_scratch_setup(device)) return rc;
     if (info) {
         memset(info, 0, sizeof(*info));
         strncpy(info->name, p.name, sizeof(info->name) - 1);

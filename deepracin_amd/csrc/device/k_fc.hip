@@ -181,6 +181,26 @@ fc_permute_rows_kernel(const float* __restrict__ src, float* __restrict__ dst, i
     for (int n = threadIdx.x; n < N; n += blockDim.x) dst[drow + n] = src[srow + n];
 }
 
+// Partial sums of drhip_fc_noalloc_f32: device memory that exists from the moment the code object
+// is loaded until the process ends (one copy per GPU), so that entry point never allocates.
+constexpr size_t kFcStaticScratchFloats = 256 * 1024;      // 1 MiB
+static __device__ __align__(256) float fc_static_scratch[kFcStaticScratchFloats];
+
+constexpr int kFcMaxDevices = 64;
+static float* g_fc_static_ptr[kFcMaxDevices];              // device address of the array on each GPU, set by drhip_init
+
+// Called by drhip_init with `device` current: looks up where this GPU holds fc_static_scratch.
+// The array's name is only a host-side handle; kernels and copies must be given this address.
+int fc_static_scratch_setup(int device) {
+    if (device < 0 || device >= kFcMaxDevices) return fail(DRHIP_EINVAL, "device ordinal %d beyond the %d this library keeps scratch for", device, kFcMaxDevices);
+    if (g_fc_static_ptr[device]) return DRHIP_OK;
+    float* p = nullptr;
+    if (int rc = check(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(fc_static_scratch)), "hipGetSymbolAddress(fc_static_scratch)")) return rc;
+    if (!p) return fail(DRHIP_EDEVICE, "hipGetSymbolAddress(fc_static_scratch) returned a NULL address");
+    g_fc_static_ptr[device] = p;
+    return DRHIP_OK;
+}
+
 }  // namespace drhip
 
 using namespace drhip;
@@ -250,4 +270,23 @@ extern "C" int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, in
     DRHIP_REQUIRE((long long)W * H * C < (1ll << 31), "drhip_fc_permute_rows_f32: K too large");
     launch(fc_permute_rows_kernel, dim3(W * H * C), dim3(256), 0, as_stream(stream), src, dst, W, H, C, N);
     return launched("fc_permute_rows_kernel");
+}
+
+extern "C" size_t drhip_fc_noalloc_max_scratch_floats(void) { return kFcStaticScratchFloats; }
+
+extern "C" int drhip_fc_noalloc_f32(const float* x, const float* Wt, const float* bias, float* y,
+                                    int K, int N, int relu, void* stream) {
+    DRHIP_REQUIRE(x && Wt && y, "drhip_fc_noalloc_f32: NULL pointer");
+    DRHIP_REQUIRE(K > 0 && N > 0, "drhip_fc_noalloc_f32: bad shape K=%d N=%d", K, N);
+    const size_t need = drhip_fc_scratch_floats(K, N);
+    DRHIP_REQUIRE(need <= kFcStaticScratchFloats,
+                  "drhip_fc_noalloc_f32: K=%d N=%d needs %zu floats of partial sums, the built-in scratch holds %zu; use drhip_fc_f32 with a caller buffer",
+                  K, N, need, kFcStaticScratchFloats);
+    DRHIP_REQUIRE(!launch_timer().on, "drhip_fc_noalloc_f32: not available between drhip_timing_begin and drhip_timing_end (timing creates events)");
+    int device = -1;
+    if (int rc = check(hipGetDevice(&device), "hipGetDevice")) return rc;
+    DRHIP_REQUIRE(device >= 0 && device < kFcMaxDevices && g_fc_static_ptr[device],
+                  "drhip_fc_noalloc_f32: drhip_init has not been called for device %d", device);
+    // The partial sums need no clearing: every (slice, column) the finishing kernel reads is written by this call's GEMV.
+    return drhip_fc_ex_f32(x, nullptr, Wt, bias, y, need ? g_fc_static_ptr[device] : nullptr, K, N, relu, 0, stream);
 }

@@ -202,6 +202,19 @@ typedef struct drhip_deferred_vec {
 int drhip_fc_slices(int K, int N);
 int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, const float* Wt, const float* bias, float* y,
                     float* partials, int K, int N, int relu, int defer, void* stream);
+/* drhip_fc_f32 for callers that cannot allocate device memory and have none to lend (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same result, bit for bit, as drhip_fc_f32; the partial sums live in a 1 MiB array that
+ * is part of the library's code object (one copy per GPU, held until the process ends, its address
+ * looked up by drhip_init, which must have run for the current device).  The call allocates and
+ * frees nothing.  Shapes whose partial sums exceed drhip_fc_noalloc_max_scratch_floats() floats
+ * (drhip_fc_scratch_floats(K,N) tells) are refused with DRHIP_EINVAL; VGG16's three layers need
+ * 229376, 131072 and 32000.  All calls on one GPU share the array: calls that may overlap (different
+ * streams, or graph branches) race on it; calls on one stream are safe.  Refused while
+ * drhip_timing_begin is active. */
+size_t drhip_fc_noalloc_max_scratch_floats(void);
+int drhip_fc_noalloc_f32(const float* x, const float* Wt, const float* bias, float* y,
+                         int K, int N, int relu, void* stream);
 /* dst[k_chw][n] = src[k_hwc][n] with k_hwc = (y*W + x)*C + z for k_chw = (z*H + y)*W + x. */
 int drhip_fc_permute_rows_f32(const float* src, float* dst, int W, int H, int C, int N, void* stream);
 
