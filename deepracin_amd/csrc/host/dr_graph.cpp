@@ -165,10 +165,14 @@ gboolean dR_setAsOutput(dR_Graph* net, dR_Node* node) {
 
 gboolean dR_prepare(dR_Graph* net) {
     const bool talk = verbose(net);
+    // One dR_prepare per graph: the schedule flags of the nodes, the planned buffers and the uploaded
+    // weights of the first call are not rolled back, so a second walk would find every node already
+    // queued and schedule nothing.  Refused loudly instead of returning a graph that computes nothing.
+    if (net->scheduledLayers || net->prepared) {
+        say("dR_prepare: this graph has been prepared already; build a new graph (dR_NewGraph) to prepare again.\n");
+        return FALSE;
+    }
     if (!ensure_device(net)) { say("dR_initCL Failed \n"); return FALSE; }
-
-    // a second dR_prepare plans new buffers: the recorded launch graph of the old ones must go
-    if (net->drGraphExec) { drhip_graph_destroy(net->drGraphExec); net->drGraphExec = NULL; }
     net->drGraphOff = FALSE;
 
     if (talk) say("Propagate shapes and schedule...\n");

@@ -39,8 +39,13 @@ bool concat_can_fuse(const dR_Node* c) {
     if (cd->concatDim != 2) return false;
     if (c->outputBuf && c->outputBuf->outputBuf) return false;  // caller-supplied storage
     std::vector<dR_Node*> ins = nodes_of(c->previous_layers);
+    int off = 0;    // floats in front of producer i inside the joint buffer
     for (size_t i = 0; i < ins.size(); ++i) {
         const dR_Node* p = ins[i];
+        // The normalization kernels move 16 bytes per lane and refuse other addresses: such a producer
+        // may only sit at a multiple of 4 floats (buffers themselves start 256-byte aligned).
+        if (p->type == tNormalization && (off & 3)) return false;
+        off += p->oshape.s0 * p->oshape.s1 * p->oshape.s2;
         if (p->type == tDataFeedNode || p->output) return false;
         if (!p->next_layers || p->next_layers->length != 1) return false;
         if (p->outputBuf) return false;     // already bound to a caller buffer

@@ -250,14 +250,23 @@ def softmax_f64(x):
 # whole networks
 # ---------------------------------------------------------------------------------------------
 
-def run_spec(spec, feeds, force_direct=False, f64=False):
+def run_spec(spec, feeds, force_direct=False, f64=False, inputs_from=None):
     """Evaluate a layer list (see deepracin_amd.configs) on the CPU.
 
     spec: list of dicts; node i may reference earlier nodes by index ('in' / 'ins').
     feeds: {node index: array [C,H,W]}.  Returns the list of all node outputs.
     f64=True evaluates with the closed forms instead of the fp32 restatements.
+    inputs_from: {node index: array}; a node that reads one of these nodes is given that array instead of
+    this evaluation's own result, so that every layer can be judged on the inputs the implementation
+    under test actually had (per-layer error without the drift of the layers in front).
     """
-    outs = []
+    class _Inputs(list):
+        def __getitem__(self, k):
+            if inputs_from is not None and k in inputs_from and spec[k]["op"] != "feed":
+                return np.asarray(inputs_from[k], np.float64 if f64 else np.float32)
+            return list.__getitem__(self, k)
+
+    outs = _Inputs()
     for idx, n in enumerate(spec):
         op = n["op"]
         if op == "feed":
@@ -291,7 +300,7 @@ def run_spec(spec, feeds, force_direct=False, f64=False):
         else:
             raise ValueError("unknown op %r" % op)
         outs.append(v)
-    return outs
+    return list(outs)
 
 
 def parse_graph_dir(path):

@@ -47,3 +47,32 @@ def rel_err(a, b):
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+RTOL, ATOL_OF_MAX = 1e-4, 1e-6
+
+
+def elem_err(a, b):
+    """Element-wise criterion: worst |a-b| / (1e-4*|b| + 1e-6*max|b|); <= 1 passes.  Unlike rel_err it does
+    not let an element of small magnitude be far off just because the layer has large elements elsewhere.
+    Returns (ratio, flat index of the worst element)."""
+    a = np.asarray(a, np.float64).reshape(-1)
+    b = np.asarray(b, np.float64).reshape(-1)
+    if a.size == 0:
+        return 0.0, -1
+    bound = RTOL * np.abs(b) + ATOL_OF_MAX * max(np.abs(b).max(), 1e-30)
+    r = np.abs(a - b) / bound
+    k = int(np.argmax(r))
+    return float(r[k]), k
+
+
+def assert_close(got, want, what="tensor", tol=RTOL):
+    """Both gates of the per-layer parity bar: max|got-want| / max|want| <= tol (norm-wise) and, element by
+    element, |got-want| <= 1e-4*|want| + 1e-6*max|want|.  The message names the worst element."""
+    got, want = np.asarray(got), np.asarray(want)
+    assert got.shape == want.shape, "%s: shape %s vs %s" % (what, got.shape, want.shape)
+    e = rel_err(got, want)
+    r, k = elem_err(got, want)
+    msg = "%s: norm-wise %.3g; worst element #%d got %.9g want %.9g (%.3g x its bound)" % (
+        what, e, k, got.reshape(-1)[k] if k >= 0 else 0.0, want.reshape(-1)[k] if k >= 0 else 0.0, r)
+    assert e <= tol and r <= 1.0, msg

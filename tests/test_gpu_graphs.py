@@ -13,7 +13,7 @@ import pytest
 
 import deepracin_amd as dr
 from deepracin_amd import configs
-from conftest import GOLDEN, rel_err
+from conftest import GOLDEN, assert_close, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -73,11 +73,20 @@ def all_compute_nodes(spec, outs):
 
 
 def check_layers(oracle, spec, feeds, got, force_direct=False):
+    """Two comparisons with the oracle.  End to end (the oracle's own chain of layers): norm-wise 1e-4 per
+    node.  Layer by layer (the oracle evaluates every node on the tensors the GPU produced for its
+    inputs): norm-wise 1e-4 and element-wise |gpu-oracle| <= 1e-4*|oracle| + 1e-6*max|oracle| -- applied
+    to the nodes all of whose inputs are feeds or downloaded tensors."""
     want = oracle.run_spec(spec, feeds, force_direct=force_direct)
     for i, g in got.items():
         assert g.shape == want[i].shape, "node %d shape %s vs %s" % (i, g.shape, want[i].shape)
         e = rel_err(g, want[i])
         assert e <= LAYER_TOL, "node %d (%s): rel err %.3g" % (i, spec[i]["op"], e)
+    step = oracle.run_spec(spec, feeds, force_direct=force_direct, inputs_from=got)
+    for i, g in got.items():
+        ins = spec[i].get("ins", [spec[i]["in"]] if "in" in spec[i] else [])
+        if all(j in got or spec[j]["op"] == "feed" for j in ins):
+            assert_close(g, step[i], "node %d (%s) on the GPU's own inputs" % (i, spec[i]["op"]), LAYER_TOL)
     return want
 
 
@@ -124,7 +133,7 @@ def test_maxpool_fused_into_convolution(oracle, gpu):
     _, _, plain = run_config("vgg_conv3", env_vars={"DR_FUSE_POOL": "0"})
     assert np.array_equal(fused[4], plain[4]) and fused[4].shape == (256, 28, 28)
     want = oracle.run_spec(spec, feeds)
-    assert rel_err(fused[4], want[4]) <= LAYER_TOL
+    assert_close(fused[4], want[4], "fused pool")
     # the pooling node of the fused run launches nothing
     with dr.Environment() as env:
         g = env.create_graph()
@@ -179,7 +188,7 @@ def test_fc_chain_fused(oracle, gpu):
         assert g.lib.dR_apply(g.ptr) and g.lib.drhip_timing_count() == 3
     assert np.array_equal(outs[2], res["0"])
     for k in range(3):
-        assert rel_err(outs[k], want[k + 1]) <= LAYER_TOL
+        assert_close(outs[k], want[k + 1], "fc chain %d" % k)
 
 
 def test_conv_global_average_softmax_fused(oracle, gpu):
@@ -224,12 +233,38 @@ def test_squeezenet_with_normalization_node(oracle, gpu):
     assert spec[1]["op"] == "norm" and float(feeds[0].max()) > 100.0
     want = oracle.run_spec(spec, feeds)
     for i in got:
-        assert rel_err(got[i], want[i]) <= LAYER_TOL
+        assert_close(got[i], want[i], "node %d" % i)
     assert int(got[len(spec) - 1].argmax()) == int(want[-1].argmax())
     # the node alone, as an output
     _, _, only = run_config("squeezenet", outputs=[1], size=96, normalise_in_graph=True)
-    assert rel_err(only[1], want[1]) <= LAYER_TOL
+    assert_close(only[1], want[1], "normalization node")
     assert abs(float(only[1].astype(np.float64).mean())) < 1e-4 and abs(float(only[1].astype(np.float64).std()) - 1.0) < 1e-4
+
+
+def test_normalization_behind_an_odd_volume_producer_in_a_concat(oracle, gpu):
+    """feed 5x5x3 -> {1x1 conv (75 floats), Normalization} -> channel concat: a fused concat would put the
+    Normalization node 300 bytes into the buffer, where its 16-byte accesses cannot go; the graph is valid
+    in the reference (src/dR_nodes_transform.c:238-281) and must run here in either input order."""
+    rng = np.random.default_rng(5)
+    w = rng.standard_normal((3, 3, 1, 1)).astype(np.float32)
+    x = rng.standard_normal((3, 5, 5)).astype(np.float32)
+    for ins in ([1, 2], [2, 1]):
+        spec = [{"op": "feed", "shape": (5, 5, 3)},
+                {"op": "conv", "in": 0, "w": w, "b": None, "stride": (1, 1), "relu": False},
+                {"op": "norm", "in": 0, "kind": 2, "mean": 0.0, "dev": 1.0},
+                {"op": "concat", "ins": ins, "dim": 2}]
+        want = oracle.run_spec(spec, {0: x})
+        with dr.Environment() as env:
+            g = env.create_graph()
+            nodes = configs.build_graph(g, spec, [3])
+            dr.prepare(g)
+            configs.feed_chw(nodes[0], x)
+            assert g.lib.dR_apply(g.ptr)
+            got = configs.fetch_chw(g)[0]
+            assert not g.lib.dR_prepare(g.ptr)               # one prepare per graph; refused, the plan stands
+            assert g.lib.dR_apply(g.ptr)
+            assert np.array_equal(configs.fetch_chw(g)[0], got)
+        assert_close(got, want[3], "concat %s" % ins)
 
 
 def test_config4_squeezenet(oracle, gpu):
@@ -456,3 +491,7 @@ def test_random_topologies(oracle, gpu, seed):
                 for i, a in zip(outs, got):
                     assert a.shape == want[i].shape, (seed, i, spec[i]["op"], a.shape, want[i].shape)
                     assert rel_err(a, want[i]) <= LAYER_TOL, (seed, i, spec[i]["op"], [s["op"] for s in spec])
+                if len(outs) == len(spec) - 1:           # every tensor downloaded: judge each layer on the GPU's own inputs
+                    step = oracle.run_spec(spec, {0: x}, inputs_from=dict(zip(outs, got)))
+                    for i, a in zip(outs, got):
+                        assert_close(a, step[i], "seed %d node %d (%s) of %s" % (seed, i, spec[i]["op"], [s["op"] for s in spec]))

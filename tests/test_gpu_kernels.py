@@ -9,7 +9,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from conftest import rel_err
+from conftest import assert_close, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -77,11 +77,11 @@ def test_conv_direct(lib, dev, oracle, W, H, I, O, k, s):
     out = dev.empty(want.size)
     ok(lib, lib.drhip_conv2d_direct_f32(dev.put(x), dev.put(w), dev.put(b), out, W, H, I, O, k, k, s, s, 1, None))
     got = dev.get(out, want.shape)
-    assert rel_err(got, want) <= TOL
+    assert_close(got, want)
     # linear, no bias
     want2 = oracle.conv_direct(x, w, None, (s, s), relu=False)
     ok(lib, lib.drhip_conv2d_direct_f32(dev.put(x), dev.put(w), None, out, W, H, I, O, k, k, s, s, 0, None))
-    assert rel_err(dev.get(out, want2.shape), want2) <= TOL
+    assert_close(dev.get(out, want2.shape), want2)
 
 
 @pytest.mark.parametrize("W,H,I,O,sx,sy", [(224, 224, 3, 64, 2, 2), (33, 31, 3, 9, 2, 2), (17, 13, 1, 5, 1, 1), (20, 18, 4, 70, 1, 2),
@@ -96,12 +96,12 @@ def test_first_layer_conv_with_maxpool(lib, dev, oracle, W, H, I, O, sx, sy, rel
     out = dev.empty(want.size)
     ok(lib, lib.drhip_conv3x3_pool3s2_f32(dev.put(x), dev.put(w), dev.put(b), out, W, H, I, O, sx, sy, relu, None))
     got = dev.get(out, want.shape)
-    assert rel_err(got, want) <= TOL
-    assert rel_err(got, oracle.pool_f64(oracle.conv_f64(x, w, b, stride=(sx, sy), relu=bool(relu)), (3, 3, 1), (2, 2, 1), 0)) <= TOL
+    assert_close(got, want)
+    assert_close(got, oracle.pool_f64(oracle.conv_f64(x, w, b, stride=(sx, sy), relu=bool(relu)), (3, 3, 1), (2, 2, 1), 0))
     # no bias
     want2 = oracle.pool(oracle.conv_direct(x, w, None, (sx, sy), relu=bool(relu)), (3, 3, 1), (2, 2, 1), 0)
     ok(lib, lib.drhip_conv3x3_pool3s2_f32(dev.put(x), dev.put(w), None, out, W, H, I, O, sx, sy, relu, None))
-    assert rel_err(dev.get(out, want2.shape), want2) <= TOL
+    assert_close(dev.get(out, want2.shape), want2)
     assert lib.drhip_conv3x3_pool3s2_f32(dev.put(x), dev.put(w), None, out, W, H, 5, O, sx, sy, relu, None) == -1
 
 
@@ -115,7 +115,7 @@ def test_conv_direct_valu_kernels(lib, dev, oracle):
             want = oracle.conv_direct(x, w, b, (s, s), relu=True)
             out = dev.empty(want.size)
             ok(lib, lib.drhip_conv2d_direct_f32(dev.put(x), dev.put(w), dev.put(b), out, W, H, I, O, 3, 3, s, s, 1, None))
-            assert rel_err(dev.get(out, want.shape), want) <= TOL
+            assert_close(dev.get(out, want.shape), want)
     finally:
         os.environ.pop("DR_DIRECT_VALU", None)
 
@@ -165,13 +165,13 @@ def test_winograd_conv(lib, dev, oracle, variant, W, H, I, O):
     for _ in range(2):                       # twice: a split layer must leave its counters at zero
         ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, out, W, H, I, O, 1, variant, ws, None))
         got = dev.get(out, want.shape)
-        assert rel_err(got, want) <= TOL
+        assert_close(got, want)
     truth = oracle.conv_f64(x, w, b, relu=True)
-    assert rel_err(got, truth) <= TOL
+    assert_close(got, truth)
     # linear, no bias (pre-activation values, sign-sensitive)
     want2 = oracle.conv_winograd(x, w, None, relu=False)
     ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, None, out, W, H, I, O, 0, variant, ws, None))
-    assert rel_err(dev.get(out, want2.shape), want2) <= TOL
+    assert_close(dev.get(out, want2.shape), want2)
 
 
 @pytest.mark.parametrize("variant", [1, 2, 0x11, 0x22, 0x101, 0x112])
@@ -191,7 +191,7 @@ def test_winograd_fused_maxpool(lib, dev, oracle, variant, W, H, I, O):
         ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, pooled, W, H, I, O, relu | 2, variant, ws, None))
         assert np.array_equal(dev.get(pooled, want.shape), want)
         ref = oracle.pool(oracle.conv_winograd(x, w, b, relu=bool(relu)), (2, 2, 1), (2, 2, 1), 0)
-        assert rel_err(dev.get(pooled, want.shape), ref) <= TOL
+        assert_close(dev.get(pooled, want.shape), ref)
     p = dev.empty(64)
     assert lib.drhip_conv3x3_winograd_f32(p, U, None, p, 3, 4, I, O, 2, 1, None, None) == -1      # odd width
     assert lib.drhip_conv3x3_winograd_f32(p, U, None, p, 4, 4, I, O, 4, 1, None, None) == -1      # unknown flag
@@ -206,10 +206,10 @@ def test_winograd_auto_variant_vgg_shapes(lib, dev, oracle):
         want = oracle.conv_winograd(x, w, b, relu=True)
         out = dev.empty(want.size)
         ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, W, I, O, 1, variant, ws, None))
-        assert rel_err(dev.get(out, want.shape), want) <= TOL
+        assert_close(dev.get(out, want.shape), want)
         # variant 0 without a workspace falls back to an unsplit configuration
         ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, W, I, O, 1, 0, None, None))
-        assert rel_err(dev.get(out, want.shape), want) <= TOL
+        assert_close(dev.get(out, want.shape), want)
         dev.close()
 
 
@@ -230,10 +230,10 @@ def test_conv1x1(lib, dev, oracle, variant, P, I, O):
     want = oracle.conv1x1(x, w, b, relu=True)
     out = dev.empty(want.size)
     ok(lib, lib.drhip_conv1x1_f32(dev.put(x), dev.put(w), dev.put(b), out, P, I, O, 1, variant, None))
-    assert rel_err(dev.get(out, want.shape), want) <= TOL
+    assert_close(dev.get(out, want.shape), want)
     want2 = oracle.conv1x1(x, w, None, relu=False)
     ok(lib, lib.drhip_conv1x1_f32(dev.put(x), dev.put(w), None, out, P, I, O, 0, variant, None))
-    assert rel_err(dev.get(out, want2.shape), want2) <= TOL
+    assert_close(dev.get(out, want2.shape), want2)
 
 
 @pytest.mark.parametrize("W,H,C,k,s", [(56, 56, 256, 2, 2), (112, 112, 64, 3, 2), (55, 55, 7, 3, 2), (14, 14, 1000, 14, 14), (9, 7, 3, 2, 3), (5, 5, 2, 5, 1),
@@ -278,7 +278,8 @@ def test_fc(lib, dev, oracle, C, H, W, N, relu):
     for _ in range(2):                     # the scratch needs no reset between calls
         ok(lib, lib.drhip_fc_f32(xd, perm, bd, y, parts, K, N, relu, None))
         got = dev.get(y, (N,))
-        assert rel_err(got, want) <= TOL and rel_err(got, truth) <= TOL
+        assert_close(got, want)
+        assert_close(got, truth)
         assert first is None or np.array_equal(first, got)      # fixed summation order
         first = got
 
@@ -306,7 +307,7 @@ def test_fc_chain_without_finishing_kernels(lib, dev, oracle, N2):
     ok(lib, lib.drhip_fc_f32(y1, W2d, b2d, y2, p2, N1, N2, 0, None))
     ok(lib, lib.drhip_softmax_f32(y2, prob, N2, None))
     want1, want2, wantp = dev.get(y1, (N1,)), dev.get(y2, (N2,)), dev.get(prob, (N2,))
-    assert rel_err(want2, oracle.fc(oracle.fc(x.reshape(K, 1, 1), W1, b1, relu=True), W2, b2, relu=False).reshape(-1)) <= TOL
+    assert_close(want2, oracle.fc(oracle.fc(x.reshape(K, 1, 1), W1, b1, relu=True), W2, b2, relu=False).reshape(-1))
     # deferred chain: y1 and y2 are never written
     q1, q2, prob2 = dev.empty(s1 * N1), dev.empty(s2 * N2), dev.empty(N2)
     ok(lib, lib.drhip_fc_ex_f32(xd, None, W1d, b1d, None, q1, K, N1, 1, 1, None))
@@ -346,12 +347,12 @@ def test_conv1x1_with_global_average(lib, dev, oracle, P, I, O, relu):
     parts = dev.empty(slices * O)
     ok(lib, lib.drhip_conv1x1_poolsum_f32(dev.put(x), dev.put(w), dev.put(b), parts, P, I, O, relu, None))
     got = dev.get(parts, (slices, O)).astype(np.float64).sum(axis=0) / P
-    assert rel_err(got, pooled) <= TOL
+    assert_close(got, pooled)
     fin, prob = dev.empty(O), dev.empty(O)
     d = DeferredVec(parts.value, None, slices, O, 0, fin.value, float(P))
     ok(lib, lib.drhip_softmax_ex_f32(None, ctypes.byref(d), prob, O, None))
-    assert rel_err(dev.get(fin, (O,)), pooled) <= TOL
-    assert rel_err(dev.get(prob, (O,)), oracle.softmax(pooled)) <= TOL
+    assert_close(dev.get(fin, (O,)), pooled)
+    assert_close(dev.get(prob, (O,)), oracle.softmax(pooled))
 
 
 @pytest.mark.parametrize("C,H,W", [(3, 224, 224), (1, 5, 7), (4, 17, 33), (64, 56, 56), (1, 1, 2)])
@@ -367,8 +368,8 @@ def test_normalize(lib, dev, oracle, C, H, W):
             got = dev.get(y, x.shape)
             assert first is None or np.array_equal(first, got)
             first = got
-        assert rel_err(got, oracle.normalize(x, kind, tm, td)) <= TOL
-        assert rel_err(got, oracle.normalize_f64(x, kind, tm, td)) <= TOL
+        assert_close(got, oracle.normalize(x, kind, tm, td))
+        assert_close(got, oracle.normalize_f64(x, kind, tm, td))
     assert lib.drhip_normalize_f32(xd, y, n, 3, 0.0, 1.0, scratch, None) == -1
     assert lib.drhip_normalize_f32(xd, y, 0, 2, 0.0, 1.0, scratch, None) == -1
 
@@ -379,14 +380,14 @@ def test_softmax(lib, dev, oracle):
         y = dev.empty(n)
         ok(lib, lib.drhip_softmax_f32(dev.put(x), y, n, None))
         got = dev.get(y, (n,))
-        assert rel_err(got, oracle.softmax(x)) <= TOL
-        assert rel_err(got, oracle.softmax_f64(x)) <= TOL
+        assert_close(got, oracle.softmax(x))
+        assert_close(got, oracle.softmax_f64(x))
         assert abs(float(got.sum()) - 1) < 1e-5 and int(got.argmax()) == int(x.argmax())
     # logits that overflow exp() unshifted still give a distribution here
     big = np.array([100.0, 101.0, 99.0], np.float32)
     y = dev.empty(3)
     ok(lib, lib.drhip_softmax_f32(dev.put(big), y, 3, None))
-    assert rel_err(dev.get(y, (3,)), oracle.softmax_f64(big)) <= TOL
+    assert_close(dev.get(y, (3,)), oracle.softmax_f64(big))
 
 
 def test_copy3d_and_scalar(lib, dev, oracle):
@@ -423,7 +424,8 @@ def test_winograd_sweep(lib, dev, oracle, W, H, I, O, variant):
     out = dev.empty(want.size)
     ok(lib, lib.drhip_conv3x3_winograd_f32(dev.put(x), U, dev.put(b), out, W, H, I, O, relu, variant, ws, None))
     got = dev.get(out, want.shape)
-    assert rel_err(got, want) <= TOL and rel_err(got, oracle.conv_f64(x, w, b, relu=bool(relu))) <= TOL
+    assert_close(got, want)
+    assert_close(got, oracle.conv_f64(x, w, b, relu=bool(relu)))
 
 
 @pytest.mark.parametrize("W,H,I,O,kw,kh,sx,sy", _sweep(12, 20, lambda r: (
@@ -437,7 +439,8 @@ def test_conv_direct_sweep(lib, dev, oracle, W, H, I, O, kw, kh, sx, sy):
     out = dev.empty(want.size)
     ok(lib, lib.drhip_conv2d_direct_f32(dev.put(x), dev.put(w), dev.put(b), out, W, H, I, O, kw, kh, sx, sy, 0, None))
     got = dev.get(out, want.shape)
-    assert rel_err(got, want) <= TOL and rel_err(got, oracle.conv_f64(x, w, b, stride=(sx, sy))) <= TOL
+    assert_close(got, want)
+    assert_close(got, oracle.conv_f64(x, w, b, stride=(sx, sy)))
 
 
 @pytest.mark.parametrize("P,I,O,variant", _sweep(13, 20, lambda r: (
@@ -447,7 +450,7 @@ def test_conv1x1_sweep(lib, dev, oracle, P, I, O, variant):
     want = oracle.conv1x1(x, w, b, relu=False)
     out = dev.empty(want.size)
     ok(lib, lib.drhip_conv1x1_f32(dev.put(x), dev.put(w), dev.put(b), out, P, I, O, 0, variant, None))
-    assert rel_err(dev.get(out, want.shape), want) <= TOL
+    assert_close(dev.get(out, want.shape), want)
 
 
 @pytest.mark.parametrize("W,H,C,kx,ky,kz,sx,sy,sz", _sweep(14, 24, lambda r: (
@@ -480,4 +483,5 @@ def test_fc_sweep(lib, dev, oracle, C, H, W, N):
     y = dev.empty(N)
     ok(lib, lib.drhip_fc_f32(dev.put(x), perm, dev.put(b), y, dev.empty(n) if n else None, K, N, 0, None))
     got = dev.get(y, (N,))
-    assert rel_err(got, want) <= TOL and rel_err(got, oracle.fc_f64(x, Wt, b).reshape(-1)) <= TOL
+    assert_close(got, want)
+    assert_close(got, oracle.fc_f64(x, Wt, b).reshape(-1))

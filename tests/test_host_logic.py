@@ -382,6 +382,51 @@ def test_schedule_order_and_buffer_plan(lib, oracle, name):
         assert len({p[0] for p in plan}) < len(spec) // 2
 
 
+def _odd_offset_norm_spec():
+    """feed 5x5x3 -> {1x1 conv to 3 channels (75 floats), Normalization} -> channel concat."""
+    rng = np.random.default_rng(5)
+    w = rng.standard_normal((3, 3, 1, 1)).astype(np.float32)
+    spec = [{"op": "feed", "shape": (5, 5, 3)},
+            {"op": "conv", "in": 0, "w": w, "b": None, "stride": (1, 1), "relu": False},
+            {"op": "norm", "in": 0, "kind": 2, "mean": 0.0, "dev": 1.0},
+            {"op": "concat", "ins": [1, 2], "dim": 2}]
+    x = rng.standard_normal((3, 5, 5)).astype(np.float32)
+    return spec, x
+
+
+def test_normalization_is_never_planned_at_an_unaligned_concat_offset(lib):
+    """The normalization kernels move 16 bytes per lane.  Behind a producer of 75 floats the fused concat
+    would put the Normalization node at byte offset 300: the planner must not fuse such a concat (and may
+    fuse it when the normalization comes first, at offset 0)."""
+    spec, _ = _odd_offset_norm_spec()
+    for ins, fused in (([1, 2], False), ([2, 1], True)):
+        spec[3] = {"op": "concat", "ins": ins, "dim": 2}
+        with dr.Environment() as env:
+            g = env.create_graph()
+            nodes = configs.build_graph(g, spec, [3])
+            assert lib.dR_propagateShapesAndSchedule(g.ptr) == 1 and lib.dR_planBuffers(g.ptr) == 1
+            plan = plan_of(g, nodes)
+        assert (plan[2][0] == plan[3][0]) == fused
+        if plan[2][0] == plan[3][0]:
+            assert plan[2][1] % 4 == 0
+
+
+def test_second_prepare_is_refused_not_silently_empty(lib, capfd):
+    """A graph is prepared once.  A second walk would find every node already queued and schedule nothing:
+    the call must say so and return FALSE, and the first schedule must still stand."""
+    spec, _, outs = configs.CONFIGS["fire"](seed=3)
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes = configs.build_graph(g, spec, outs)
+        assert lib.dR_propagateShapesAndSchedule(g.ptr) == 1
+        first = [dr.node_struct(n).drSchedulePos for n in nodes]
+        capfd.readouterr()
+        assert lib.dR_prepare(g.ptr) == 0
+        out = capfd.readouterr().out
+        assert "prepared already" in out
+        assert [dr.node_struct(n).drSchedulePos for n in nodes] == first
+
+
 # ---------------------------------------------------------------------------------------------
 # list cursor rules and helpers
 # ---------------------------------------------------------------------------------------------

@@ -176,6 +176,30 @@ def test_pool_matches_torch_on_zero_padded_input(oracle, H, W, k, s):
     assert np.allclose(got_avg, oracle.pool_f64(x, (k, k, 1), (s, s, 1), 1), rtol=1e-6)
 
 
+@pytest.mark.parametrize("C,H,W,win,st", [(8, 6, 6, (2, 2, 2), (2, 2, 2)), (7, 5, 9, (3, 2, 3), (2, 2, 2)),
+                                          (6, 4, 4, (1, 1, 3), (1, 1, 1)), (5, 7, 3, (2, 3, 2), (1, 2, 3))])
+def test_pool_with_depth_window_matches_torch_3d(oracle, C, H, W, win, st):
+    """Windows that span channels (sz > 1): torch's max_pool3d / avg_pool3d on the input zero-padded at the
+    far end of every axis are the library routines this reduces to (window anchored at out*stride, samples
+    outside read 0.0, the average divides by the full window).  A window walking the wrong axis, a stride
+    applied to the wrong axis or a divisor that forgets sz would fail."""
+    sx, sy, sz = win
+    stx, sty, stz = st
+    x = np.abs(rnd(C, H, W)) + 0.1       # positive: zero padding == -inf padding for max
+    Co, Ho, Wo = -(-C // stz), -(-H // sty), -(-W // stx)
+    padded = np.zeros((max(C, (Co - 1) * stz + sz), max(H, (Ho - 1) * sty + sy), max(W, (Wo - 1) * stx + sx)), np.float32)
+    padded[:C, :H, :W] = x
+    t = torch.from_numpy(padded)[None, None]
+    mx = F.max_pool3d(t, (sz, sy, sx), (stz, sty, stx))[0, 0].numpy()
+    av = F.avg_pool3d(t.double(), (sz, sy, sx), (stz, sty, stx))[0, 0].numpy()
+    got_max, arg = oracle.pool(x, win, st, 0, want_argmax=True)
+    got_avg = oracle.pool(x, win, st, 1)
+    assert got_max.shape == (Co, Ho, Wo) == mx.shape
+    assert np.array_equal(got_max, mx)
+    assert np.array_equal(x.reshape(-1)[arg.reshape(-1)], got_max.reshape(-1))      # the index points at the maximum
+    assert np.allclose(got_avg, av, rtol=1e-6, atol=1e-7)
+
+
 def test_pool_max_pads_with_zero_not_minus_inf(oracle):
     # a window hanging over the border sees 0.0f: with negative inputs the result is 0, not the max
     x = -np.ones((1, 3, 3), np.float32)
@@ -249,6 +273,17 @@ def test_scalar_concat_slice(oracle):
     x = rnd(4, 3, 5)
     assert np.array_equal(oracle.scalar_op(x, 1, 2.5), x - np.float32(2.5))
     assert np.array_equal(oracle.scalar_op(x, 0, 2.5), x + np.float32(2.5))
+    # the remaining operations of dR_ElemWise1OperationType against numpy's float32 routines
+    # (Kernels/dR_math.cl:170-341): 2 x*s, 3 x/s, 4 log x, 5 exp x, 6 sqrt x, 7 s, 8 pow(x, s)
+    assert np.array_equal(oracle.scalar_op(x, 2, -1.75), x * np.float32(-1.75))
+    assert np.array_equal(oracle.scalar_op(x, 3, 3.0), x / np.float32(3.0))
+    assert np.array_equal(oracle.scalar_op(x, 7, 0.625), np.full_like(x, 0.625))
+    pos = np.abs(x) + np.float32(0.5)
+    assert np.allclose(oracle.scalar_op(pos, 4, 0.0), np.log(pos.astype(np.float64)), rtol=1e-6, atol=1e-7)
+    assert np.allclose(oracle.scalar_op(x, 5, 0.0), np.exp(x.astype(np.float64)), rtol=1e-6)
+    assert np.allclose(oracle.scalar_op(pos, 6, 0.0), np.sqrt(pos.astype(np.float64)), rtol=1e-6)
+    assert np.allclose(oracle.scalar_op(pos, 8, 1.5), pos.astype(np.float64) ** 1.5, rtol=1e-6)
+    assert not np.array_equal(oracle.scalar_op(x, 3, 3.0), np.float32(3.0) / x)         # x/s, not s/x
     assert np.array_equal(oracle.slice3d(x, (1, 0, 2), (3, 2, 1)), x[2:3, 0:2, 1:4])
     assert np.array_equal(oracle.concat([x, x * 2], 2), np.concatenate([x, x * 2], 0))
 
