@@ -140,14 +140,19 @@ __device__ inline f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset, un
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voffset, (int)soffset, 0));
 }
 
-template <int NT>
-__global__ void __launch_bounds__(kWinoThreads, (NT == 1 ? 3 : (NT == 2 ? 2 : 1)))
+// KW = 2: the workgroup has eight waves; waves 4..7 repeat the roles of waves 0..3 on every second stage
+// (wave set k takes the stages chBegin + k, + KW, ...), and the two sets' sums meet in LDS in the epilogue,
+// set 0 first.  One wave per SIMD cannot keep the matrix pipe busy (it waits for its own transforms and
+// loads); layers whose workgroup count leaves one workgroup per CU get their second wave per SIMD this way,
+// without a second workgroup's share of partial tiles in memory.
+template <int NT, int KW>
+__global__ void __launch_bounds__(kWinoThreads * KW, KW == 2 ? 1 : (NT == 1 ? 3 : (NT == 2 ? 2 : 1)))
 winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__ U,
                          const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
                          int W, int H, int I, int O, int tilesX, int T, int nTB, int nBlocks,
                          int chunksPerSplit, int relu, int vec2) {
     constexpr int TB = 32, OB = 32 * NT, KC = kWinoKC;
-    extern __shared__ float P[];                    // epilogue only: [4 rows][2][OB o][32 t] floats
+    extern __shared__ float P[];                    // epilogue only: [KW sets][4 rows][2][OB o][32 t] floats
 
     // ---- which panel: XCD-aware remap of the linear workgroup id -----------------------------
     const int perXcd = gridDim.x / kXcds;           // grid is padded to a multiple of kXcds
@@ -158,7 +163,9 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     const int split = blockIdx.y, nSplits = gridDim.y;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // = row of the transform
+    const int waveId = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = waveId & 3;                    // = row of the transform
+    const int kset = waveId >> 2;                   // which of the KW wave sets
     const int l32 = lane & 31, lhi = lane >> 5;
     const int plane = H * W;
     const int nChunksAll = (I + KC - 1) / KC;
@@ -218,10 +225,11 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     // The epilogue's bias values are fetched now: a load issued there would add a trip to memory
     // to the tail of every workgroup.
     constexpr bool kBiasEarly = NT <= 2;
-    float biasEarly[kBiasEarly ? OB / 8 : 1];
+    constexpr int EO = 8 * KW;                      // output channels finished per pass of the epilogue
+    float biasEarly[kBiasEarly ? OB / EO : 1];
     if (kBiasEarly && bias && gridDim.y == 1) {
 #pragma unroll
-        for (int q = 0; q < OB / 8; ++q) biasEarly[q] = bias[min(o0 + (tid >> 5) + 8 * q, O - 1)];
+        for (int q = 0; q < OB / EO; ++q) biasEarly[q] = bias[min(o0 + (tid >> 5) + EO * q, O - 1)];
     }
 
     f32x16 acc[4][NT];
@@ -235,14 +243,14 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     float raw[4][8];
     f32x4 f[4][NT];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) load_rows_ranged(raw[ks], chBegin * KC + 2 * ks);
+    for (int ks = 0; ks < 4; ++ks) load_rows_ranged(raw[ks], (chBegin + kset) * KC + 2 * ks);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) load_filters(f[e], e, chBegin);
+    for (int e = 0; e < 4; ++e) load_filters(f[e], e, min(chBegin + kset, nChunksAll - 1));
 
     // One stage: transform the rows of chunk ch (and start loading those of chunk ch+1 into the
     // same registers), then 16*NT MFMAs, reloading the filters of each xi pair behind its MFMAs.
     auto stage = [&](int ch, auto plainNext) {
-        const int next = min(ch + 1, nChunksAll - 1);
+        const int next = min(ch + KW, nChunksAll - 1);
         float b[4][4];                              // [k-step][xi within the row]
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
@@ -274,8 +282,8 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
                     for (int nt = 0; nt < NT; ++nt)
                         acc[e][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[e][nt][ks], b[ks][e], acc[e][nt], 0, 0, 0);
                 if (eg == 0) {
-                    if constexpr (decltype(plainNext)::value) load_rows_plain(raw[ks], (ch + 1) * KC + 2 * ks);
-                    else load_rows_ranged(raw[ks], (ch + 1) * KC + 2 * ks);
+                    if constexpr (decltype(plainNext)::value) load_rows_plain(raw[ks], (ch + KW) * KC + 2 * ks);
+                    else load_rows_ranged(raw[ks], (ch + KW) * KC + 2 * ks);
                 } else if (ks < 2) {
                     load_filters(f[ks], ks, next);
                 }
@@ -286,12 +294,12 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
         load_filters(f[3], 3, next);
         __builtin_amdgcn_sched_barrier(0);
     };
-    // Stages whose successor chunk is complete (all 8 channels exist) prefetch in the plain form;
-    // the last one or two of the tensor use the ranged form.
-    const int chMain = max(chBegin, min(chEnd, I / KC - 1));
-    int ch = chBegin;
-    for (; ch < chMain; ++ch) stage(ch, std::true_type{});
-    for (; ch < chEnd; ++ch) stage(ch, std::false_type{});
+    // Stages whose successor chunk (KW further on) is complete (all 8 channels exist) prefetch in the
+    // plain form; the last ones of the tensor use the ranged form.
+    const int chMain = min(chEnd, I / KC - KW);
+    int ch = chBegin + kset;
+    for (; ch < chMain; ch += KW) stage(ch, std::true_type{});
+    for (; ch < chEnd; ch += KW) stage(ch, std::false_type{});
 
     // ---- epilogue -----------------------------------------------------------------------------
     // Accumulator layout of the 32x32 MFMA: lane -> column (tile) lane%32; register r -> row
@@ -304,8 +312,8 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
         for (int r = 0; r < 16; ++r) {
             const float m0 = acc[0][nt][r], m1 = acc[1][nt][r], m2 = acc[2][nt][r], m3 = acc[3][nt][r];
             const int ol = 32 * nt + 8 * (r / 4) + 4 * lhi + (r % 4);
-            P[((wave * 2 + 0) * OB + ol) * TB + l32] = m0 + m1 + m2;
-            P[((wave * 2 + 1) * OB + ol) * TB + l32] = m1 - m2 + m3;
+            P[(((kset * 4 + wave) * 2 + 0) * OB + ol) * TB + l32] = m0 + m1 + m2;
+            P[(((kset * 4 + wave) * 2 + 1) * OB + ol) * TB + l32] = m1 - m2 + m3;
         }
     }
     // LDS-only barrier: __syncthreads() would also wait for the outstanding (unused) prefetches.
@@ -313,7 +321,7 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 
-    // Left factor A^T over the four rows, bias, ReLU, store: lane -> tile tid%32, channels tid/32 + 8q.
+    // Left factor A^T over the four rows, bias, ReLU, store: lane -> tile tid%32, channels tid/32 + EO*q.
     const bool direct = nSplits == 1;
     const int et = tid & 31, eo = tid >> 5;
     const int etg = t0 + et;
@@ -321,13 +329,17 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     const int ox = eTileOk ? 2 * (etg % tilesX) : 0, oy = eTileOk ? 2 * (etg / tilesX) : 0;
     f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
 #pragma unroll
-    for (int q = 0; q < OB / 8; ++q) {
-        const int ol = eo + 8 * q, o = o0 + ol;
+    for (int q = 0; q < OB / EO; ++q) {
+        const int ol = eo + EO * q, o = o0 + ol;
         float p[4][2];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             p[r][0] = P[((r * 2 + 0) * OB + ol) * TB + et];
             p[r][1] = P[((r * 2 + 1) * OB + ol) * TB + et];
+            if constexpr (KW == 2) {                // the second wave set's half of the channel sum
+                p[r][0] += P[(((4 + r) * 2 + 0) * OB + ol) * TB + et];
+                p[r][1] += P[(((4 + r) * 2 + 1) * OB + ol) * TB + et];
+            }
         }
         float y00 = p[0][0] + p[1][0] + p[2][0], y01 = p[0][1] + p[1][1] + p[2][1];
         float y10 = p[1][0] - p[2][0] + p[3][0], y11 = p[1][1] - p[2][1] + p[3][1];
@@ -574,9 +586,13 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
 // variant = output channels per workgroup (low 4 bits: 1 -> 32, 2 -> 64, 3 -> 128)
 //         | log2(number of input-channel splits) << 4
 //         | 0x100: 16-tile blocks (then the low 4 bits mean 1 -> 16, 2 -> 32, 3 -> 64 channels)
-struct WinoCfg { int nt, splits, tb; };
+//         | 0x400: eight waves per workgroup, two wave sets sharing the stages (32-tile blocks of 32 or 64 channels)
+struct WinoCfg { int nt, splits, tb, waveSets; };
 
 static bool wino_variant(int variant, WinoCfg* c) {
+    c->waveSets = (variant & 0x400) ? 2 : 1;
+    if (c->waveSets == 2 && ((variant & 0x300) || (variant & 0xf) > 2)) return false;
+    variant &= ~0x400;
     const int lg = (variant >> 4) & 0xf;
     if (lg > 6 || (variant >> 9)) return false;
     c->splits = 1 << lg;
@@ -606,7 +622,6 @@ static WinoGeom wino_geom(int W, int H, int I, int O, const WinoCfg& c) {
 }
 
 // Workspace: [splits][panel][o in panel][tile in panel] partial 2x2 tiles (float4 each).
-
 template <int NT, int TB>
 static int launch_wino(const float* in, const float* U, const float* bias, float* out, float* workspace,
                        int W, int H, int I, int O, int relu, const WinoCfg& c, hipStream_t s) {
@@ -615,10 +630,25 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
     const int gridX = ceil_div(g.nBlocks, kXcds) * kXcds;
     const size_t ldsBytes = 4 * 2 * OB * TB * sizeof(float);
     const int vec2 = ((W & 1) == 0) && (((size_t)out & 7) == 0);
-    if constexpr (TB == 32)
-        launch((winograd_f23_mfma_kernel<NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
-               in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
-    else
+    if constexpr (TB == 32) {
+        if constexpr (NT <= 2) {
+            if (c.waveSets == 2) {
+                // more than 64 KiB of dynamic LDS has to be asked for once per kernel
+                static bool raised = false;
+                if (2 * ldsBytes > 65536 && !raised) {
+                    if (int rc = check(hipFuncSetAttribute((const void*)winograd_f23_mfma_kernel<NT, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * ldsBytes)),
+                                       "hipFuncSetAttribute(max dynamic LDS)")) return rc;
+                    raised = true;
+                }
+            }
+            if (c.waveSets == 2)
+                launch((winograd_f23_mfma_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
+                       in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
+        }
+        if (c.waveSets != 2 || NT > 2)
+            launch((winograd_f23_mfma_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
+                   in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
+    } else
         launch((winograd_f23_mfma16_kernel<NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
                in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
@@ -655,9 +685,12 @@ extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     int lg = 0;
     // (a split costs a second kernel: below 6 stages in all it does not pay)
     while (lg < 5 && nChunks >= 6 && (panels << lg) < (5 * cus) / 8 && (nChunks >> (lg + 1)) >= 2) ++lg;
-    // A split layer that still has 32 or more stages per split (28x28, 512 -> 512): the same number
-    // of workgroups as 64-channel panels with twice the splits share each input transform between
-    // two MFMA sets (26.1 vs 27.5 us).
+    // At most one workgroup per CU and at least two stages for each wave set: eight waves per workgroup,
+    // so that every SIMD still has two waves to alternate between (56x56 256->256: 23.6 vs 24.8 us;
+    // 28x28 512->512 as 112 panels x 2 splits: 26.3 vs 26.9 us for 64-channel panels x 4 splits).
+    if ((panels << lg) <= cus && (nChunks >> lg) >= 4) return 0x400 | code | (lg << 4);
+    // A split layer that still has 32 or more stages per split: the same number of workgroups as
+    // 64-channel panels with twice the splits share each input transform between two MFMA sets.
     if (code == 1 && lg >= 1 && lg < 5 && O >= 64 && (nChunks >> lg) >= 32) return 2 | ((lg + 1) << 4);
     return code | (lg << 4);
 }
@@ -696,7 +729,7 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
     DRHIP_REQUIRE(!(relu & DRHIP_EPILOGUE_MAXPOOL2) || ((W | H) & 1) == 0, "drhip_conv3x3_winograd_f32: the fused 2x2 max pool needs even W and H (got %dx%d)", W, H);
     if (variant == 0) {
         variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O);
-        if (!workspace) variant &= 0xf;            // no workspace offered: stay unsplit
+        if (!workspace) variant &= 0x50f;          // no workspace offered: stay unsplit
     }
     WinoCfg c;
     DRHIP_REQUIRE(wino_variant(variant, &c), "drhip_conv3x3_winograd_f32: unknown variant %d", variant);

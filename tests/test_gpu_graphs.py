@@ -13,7 +13,7 @@ import pytest
 
 import deepracin_amd as dr
 from deepracin_amd import configs
-from conftest import GOLDEN, assert_close, rel_err
+from conftest import GOLDEN, assert_close, rel_err, spec_terms
 
 pytestmark = pytest.mark.gpu
 
@@ -86,7 +86,7 @@ def check_layers(oracle, spec, feeds, got, force_direct=False):
     for i, g in got.items():
         ins = spec[i].get("ins", [spec[i]["in"]] if "in" in spec[i] else [])
         if all(j in got or spec[j]["op"] == "feed" for j in ins):
-            assert_close(g, step[i], "node %d (%s) on the GPU's own inputs" % (i, spec[i]["op"]), LAYER_TOL)
+            assert_close(g, step[i], "node %d (%s) on the GPU's own inputs" % (i, spec[i]["op"]), LAYER_TOL, spec_terms(spec[i]))
     return want
 
 
@@ -494,4 +494,5 @@ def test_random_topologies(oracle, gpu, seed):
                 if len(outs) == len(spec) - 1:           # every tensor downloaded: judge each layer on the GPU's own inputs
                     step = oracle.run_spec(spec, {0: x}, inputs_from=dict(zip(outs, got)))
                     for i, a in zip(outs, got):
-                        assert_close(a, step[i], "seed %d node %d (%s) of %s" % (seed, i, spec[i]["op"], [s["op"] for s in spec]))
+                        assert_close(a, step[i], "seed %d node %d (%s) of %s" % (seed, i, spec[i]["op"], [s["op"] for s in spec]),
+                                     terms=spec_terms(spec[i]))
