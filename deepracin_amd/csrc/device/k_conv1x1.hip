@@ -130,10 +130,23 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 constexpr int kC1Chunk = 8;         // k-steps per chunk (16 in flight was measured slower)
 constexpr int kC1Pad16 = 17;
 
-__global__ void __launch_bounds__(1024)
+// POOL: the input is the tensor IN FRONT of a 3x3 / stride-2 max pooling ([I][Hin][Win]) and the B operand of
+// pixel p = (py, px) of the pooled map is taken on load as the maximum of the window anchored at (2px, 2py),
+// samples outside the map counting as 0.0 (src/dR_nodes_pooling.c:277-401) -- the pooled tensor, read exactly
+// once by this layer, is never written and the pooling kernel in front is not launched.  A window row is ONE
+// 16-byte buffer load from its first sample (nine dword gathers per operand kept the CU's address unit busy
+// for longer than the whole unpooled layer takes); the resource ends with the tensor, so the load of the
+// last row may run past it and reads 0.0 there.  Chunks of 4 k-steps keep the rows in registers.
+typedef float f32x4ld __attribute__((ext_vector_type(4)));
+constexpr unsigned kC1BufferFlags = 0x00020000u;    // dword 3 of a gfx9 raw buffer resource (32-bit data format)
+
+template <bool POOL>
+__global__ void __launch_bounds__(POOL ? 512 : 1024)
 conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
-                      float* __restrict__ out, int P, int I, int O, int nPT, int relu) {
+                      float* __restrict__ out, int P, int I, int O, int nPT, int relu, int Win, int Hin, int Wp) {
     extern __shared__ float part[];                 // [KW][16][kC1Pad16]
+    constexpr int CH = POOL ? 4 : kC1Chunk;         // k-steps per chunk
+    constexpr int NS = POOL ? 12 : 1;               // floats loaded per B operand (3 window rows of 4)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int KW = blockDim.x >> 6;
@@ -142,27 +155,61 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
     const int nK = (I + 3) / 4;                     // k-steps of 4 channels
     const int oL = min(o0 + l16, O - 1), pL = min(p0 + l16, P - 1);
     const bool oOk = o0 + l16 < O, pOk = p0 + l16 < P;
+    const int plane = POOL ? Win * Hin : P;
+
+    // POOL: element offset of each window row inside a channel plane (rows below the map repeat the last row
+    // and are masked), and which of the 3x3 samples lie inside the map
+    int rowOff[3] = {pL, 0, 0};
+    bool colIn[3] = {true, true, true}, rowIn[3] = {true, true, true};
+    __amdgpu_buffer_rsrc_t rIn;
+    if constexpr (POOL) {
+        const int py = pL / Wp, px = pL - py * Wp;
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+            rowIn[d] = 2 * py + d < Hin;
+            colIn[d] = 2 * px + d < Win;
+            rowOff[d] = min(2 * py + d, Hin - 1) * Win + 2 * px;
+        }
+        rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kC1BufferFlags);
+    }
 
     f32x4v acc = {0.f, 0.f, 0.f, 0.f};
-    float aA[kC1Chunk], bA[kC1Chunk], aB[kC1Chunk], bB[kC1Chunk];
-    // chunk j of this wave = its k-steps wave + KW*(8j .. 8j+7)
-    auto load_chunk = [&](float (&a)[kC1Chunk], float (&b)[kC1Chunk], int j) {
+    float aA[CH], bA[CH][NS], aB[CH], bB[CH][NS];
+    // chunk j of this wave = its k-steps wave + KW*(CH*j .. CH*j + CH-1)
+    auto load_chunk = [&](float (&a)[CH], float (&b)[CH][NS], int j) {
 #pragma unroll
-        for (int u = 0; u < kC1Chunk; ++u) {
-            const int c = min(4 * (wave + KW * (kC1Chunk * j + u)) + lk, I - 1);
+        for (int u = 0; u < CH; ++u) {
+            const int c = min(4 * (wave + KW * (CH * j + u)) + lk, I - 1);
             a[u] = w[(size_t)c * O + oL];
-            b[u] = in[(size_t)c * P + pL];
+            if constexpr (POOL) {
+#pragma unroll
+                for (int d = 0; d < 3; ++d) {
+                    const f32x4ld v = __builtin_bit_cast(f32x4ld, __builtin_amdgcn_raw_buffer_load_b128(rIn, 4 * (c * plane + rowOff[d]), 0, 0));
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) b[u][4 * d + e] = v[e];
+                }
+            } else {
+                b[u][0] = in[(size_t)c * plane + rowOff[0]];
+            }
         }
     };
-    auto multiply = [&](const float (&a)[kC1Chunk], const float (&b)[kC1Chunk], int j) {
+    auto multiply = [&](const float (&a)[CH], const float (&b)[CH][NS], int j) {
 #pragma unroll
-        for (int u = 0; u < kC1Chunk; ++u) {
-            const bool cOk = 4 * (wave + KW * (kC1Chunk * j + u)) + lk < I;
-            acc = __builtin_amdgcn_mfma_f32_16x16x4f32((cOk && oOk) ? a[u] : 0.0f, (cOk && pOk) ? b[u] : 0.0f, acc, 0, 0, 0);
+        for (int u = 0; u < CH; ++u) {
+            const bool cOk = 4 * (wave + KW * (CH * j + u)) + lk < I;
+            float bv = b[u][0];
+            if constexpr (POOL) {
+                bv = -3.402823466e+38f;              // the pooling kernel's start value
+#pragma unroll
+                for (int d = 0; d < 3; ++d)
+#pragma unroll
+                    for (int e = 0; e < 3; ++e) bv = fmaxf(bv, (rowIn[d] && colIn[e]) ? b[u][4 * d + e] : 0.0f);
+            }
+            acc = __builtin_amdgcn_mfma_f32_16x16x4f32((cOk && oOk) ? a[u] : 0.0f, (cOk && pOk) ? bv : 0.0f, acc, 0, 0, 0);
         }
     };
     const int mine = (nK - wave + KW - 1) / KW;                 // k-steps of this wave (>= 0)
-    const int chunks = (mine + kC1Chunk - 1) / kC1Chunk;
+    const int chunks = (mine + CH - 1) / CH;
     // Two buffers, the next chunk always on its way.  The loop leaves right after the last real
     // chunk: the loads issued beyond it (clamped addresses) are never waited for.
     load_chunk(aA, bA, 0);
@@ -226,8 +273,8 @@ extern "C" int drhip_conv1x1_f32(const float* in, const float* w, const float* b
         DRHIP_REQUIRE((variant >> 9) == 0, "drhip_conv1x1_f32: unknown variant %#x", variant);
         DRHIP_REQUIRE(kw == 1 || kw == 2 || kw == 4 || kw == 8 || kw == 16, "drhip_conv1x1_f32: unknown variant %#x (16x16 tiles: 1..16 waves)", variant);
         const int nPT16 = ceil_div(P, 16), nOT16 = ceil_div(O, 16);
-        launch(conv1x1_mfma16_kernel, dim3(nPT16 * nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
-               in, w, bias, out, P, I, O, nPT16, relu);
+        launch(conv1x1_mfma16_kernel<false>, dim3(nPT16 * nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
+               in, w, bias, out, P, I, O, nPT16, relu, 0, 0, 0);
         return launched("conv1x1_mfma16_kernel");
     }
     DRHIP_REQUIRE(variant == 1 || variant == 2 || variant == 4 || variant == 8, "drhip_conv1x1_f32: unknown variant %d (waves per tile: 1, 2, 4, 8)", variant);
@@ -254,4 +301,21 @@ extern "C" int drhip_conv1x1_poolsum_f32(const float* in, const float* w, const 
     launch(conv1x1_mfma_kernel, dim3(nPT * nOT), dim3(64 * kw), (size_t)kw * 32 * kC1Pad * sizeof(float), as_stream(stream),
            in, w, bias, (float*)nullptr, partials, P, I, O, nPT, relu);
     return launched("conv1x1_mfma_kernel");
+}
+
+extern "C" int drhip_conv1x1_pooled3s2_f32(const float* in, const float* w, const float* bias, float* out,
+                                           int Win, int Hin, int I, int O, int relu, void* stream) {
+    DRHIP_REQUIRE(in && w && out, "drhip_conv1x1_pooled3s2_f32: NULL tensor");
+    DRHIP_REQUIRE(Win > 0 && Hin > 0 && I > 0 && O > 0, "drhip_conv1x1_pooled3s2_f32: bad shape %dx%dx%d -> %d", Win, Hin, I, O);
+    const int Wp = (Win + 1) / 2, Hp = (Hin + 1) / 2, P = Wp * Hp;
+    DRHIP_REQUIRE((long long)Win * Hin * I < (1ll << 29) && (long long)P * O < (1ll << 31) && (long long)I * O < (1ll << 31),
+                  "drhip_conv1x1_pooled3s2_f32: tensor too large for 32-bit indexing");
+    // waves per 16x16 tile: one per chunk of 4 k-steps (a single round of loads for every wave), at most 8
+    const int nK = ceil_div(I, 4);
+    int kw = 1;
+    while (kw < 8 && nK > 4 * kw) kw *= 2;
+    const int nPT16 = ceil_div(P, 16), nOT16 = ceil_div(O, 16);
+    launch(conv1x1_mfma16_kernel<true>, dim3(nPT16 * nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
+           in, w, bias, out, P, I, O, nPT16, relu, Win, Hin, Wp);
+    return launched("conv1x1_mfma16_kernel<pooled input>");
 }

@@ -183,7 +183,11 @@ gboolean conv_compute(dR_Graph* net, dR_Node* node) {
         case drConv1x1Gemm:
             if (c->drFusedAvgPool)
                 rc = drhip_conv1x1_poolsum_f32(in, w, b, (float*)c->workspaceBuf, W * H, I, O, relu, stream_of(net));
-            else
+            else if (c->drPooledInput) {        // the 3x3/2 max pooling in front is taken while loading its input
+                const dR_Pooling_Data* pd = (const dR_Pooling_Data*)c->drPooledInput->layer;
+                rc = drhip_conv1x1_pooled3s2_f32(dev_out(first_input(c->drPooledInput)), w, b, out, pd->ishape.s0, pd->ishape.s1,
+                                                 I, O, relu, stream_of(net));
+            } else
                 rc = drhip_conv1x1_f32(in, w, b, out, W * H, I, O, relu, c->variant, stream_of(net));
             break;
         default:

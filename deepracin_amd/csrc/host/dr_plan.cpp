@@ -100,6 +100,26 @@ dR_Node* pool_fusable_producer(const dR_Node* p) {
     return c;
 }
 
+// A 3x3 / stride-2 max pooling whose only reader is a 1x1 convolution: the convolution takes the window maxima
+// while it loads its input, the pooled tensor is never written and the pooling kernel is not launched
+// (DR_FUSE_POOLIN=0 keeps them apart).  Returns the pooling node in front of such a convolution.
+dR_Node* pooled_input_of(const dR_Node* c) {
+    if (c->type != tConv2d) return nullptr;
+    const char* env = getenv("DR_FUSE_POOLIN");
+    if (env && strcmp(env, "0") == 0) return nullptr;
+    const dR_Conv2d_Data* cd = (const dR_Conv2d_Data*)c->layer;
+    if (cd->algo != drConv1x1Gemm) return nullptr;
+    std::vector<dR_Node*> ins = nodes_of(c->previous_layers);
+    if (ins.size() != 1 || ins[0]->type != tPooling) return nullptr;
+    dR_Node* p = ins[0];
+    const dR_Pooling_Data* pd = (const dR_Pooling_Data*)p->layer;
+    if (pd->poolingType != tMax || pd->shape.s1 != 3 || pd->shape.s2 != 3 || pd->shape.s3 != 1) return nullptr;
+    if (pd->stride.s1 != 2 || pd->stride.s2 != 2 || pd->stride.s3 != 1) return nullptr;
+    if (p->output || p->outputBuf || !p->next_layers || p->next_layers->length != 1) return nullptr;
+    if (pool_fusable_producer(p)) return nullptr;      // already stored by the convolution in front of it
+    return p;
+}
+
 // A global average pooling (one window = the whole map) behind a 1x1 convolution and in front of an
 // FC or softmax node: the convolution's epilogue sums its pixels per tile, the consumer adds the
 // tile sums and divides, and neither the convolution's tensor nor a pooling kernel is needed
@@ -259,6 +279,8 @@ gboolean dR_planBuffers(dR_Graph* net) {
         if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drAbsorbed1x1 = ((dR_Conv2d_Data*)n->layer)->drAbsorbedBy = nullptr;
     for (dR_Node* n : sched)
         if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drFusedPool = ((dR_Conv2d_Data*)n->layer)->drFusedAvgPool = FALSE;
+    for (dR_Node* n : sched)
+        if (n->type == tConv2d) ((dR_Conv2d_Data*)n->layer)->drPooledInput = nullptr;
     for (dR_Node* n : sched) {
         if (n->type == tPooling) {
             dR_Node* c = pool_fusable_producer(n);
@@ -287,6 +309,14 @@ gboolean dR_planBuffers(dR_Graph* net) {
                 ((dR_Conv2d_Data*)ins[k]->layer)->drAbsorbedBy = ins[k + 1];
                 ((dR_Conv2d_Data*)ins[k + 1]->layer)->drAbsorbed1x1 = ins[k];
             }
+    }
+    // (after the loop above: whether a 1x1 layer feeds a fused global average is known only now)
+    for (dR_Node* n : sched) {
+        if (n->type != tConv2d || ((dR_Conv2d_Data*)n->layer)->drFusedAvgPool) continue;
+        if (dR_Node* pool = pooled_input_of(n)) {
+            ((dR_Conv2d_Data*)n->layer)->drPooledInput = pool;
+            ((dR_Pooling_Data*)pool->layer)->drFused = TRUE;
+        }
     }
     auto root_of = [&](dR_Node* n, int* offset) {
         int off = 0;
@@ -319,6 +349,13 @@ gboolean dR_planBuffers(dR_Graph* net) {
         for (dR_Node* p : nodes_of(n->previous_layers)) {
             Root& rp = touch(root_of(p, nullptr));
             rp.lastUse = std::max(rp.lastUse, n->drSchedulePos);
+        }
+        // a convolution that pools while loading reads the tensor in front of the pooling node
+        if (n->type == tConv2d && ((dR_Conv2d_Data*)n->layer)->drPooledInput) {
+            for (dR_Node* p : nodes_of(((dR_Conv2d_Data*)n->layer)->drPooledInput->previous_layers)) {
+                Root& rp = touch(root_of(p, nullptr));
+                rp.lastUse = std::max(rp.lastUse, n->drSchedulePos);
+            }
         }
     }
 

@@ -155,6 +155,16 @@ int drhip_conv1x1_f32(const float* in, const float* w, const float* bias, float*
 int drhip_conv1x1_poolsum_slices(int P);
 int drhip_conv1x1_poolsum_f32(const float* in, const float* w, const float* bias, float* partials,
                               int P, int I, int O, int relu, void* stream);
+/* A 3x3 / stride-2 max pooling followed by a 1x1 convolution, without the pooled tensor in between:
+ * in is the pooling's input [I][Hin][Win]; the convolution works on the pooled map of
+ * ceil(Win/2) x ceil(Hin/2) pixels, whose samples it takes while loading (maximum over the window
+ * anchored at (2x, 2y), samples outside the map count as 0.0); out is [O][ceil(Hin/2)][ceil(Win/2)].
+ * Same values as drhip_pool_f32 followed by drhip_conv1x1_f32 up to the rounding of a channel sum that is
+ * split over a different number of waves.  Replaces the generated
+ * pooling kernel plus `conv2d1x1` of such a pair (src/dR_nodes_pooling.c:277-401,
+ * Kernels/dR_conv2d1x1.cl:4-53). */
+int drhip_conv1x1_pooled3s2_f32(const float* in, const float* w, const float* bias, float* out,
+                                int Win, int Hin, int I, int O, int relu, void* stream);
 /* Tile configuration for a 1x1 layer (replaces dR_conv2d_1x1_schedule, :1526-1602): waves per
  * output tile (1, 2, 4, 8 for 32x32 tiles; | 0x100 = 16x16 tiles, 1..16 waves, for small layers).
  * variant 0 in drhip_conv1x1_f32 = let the launcher pick. */

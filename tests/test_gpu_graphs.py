@@ -145,6 +145,52 @@ def test_maxpool_fused_into_convolution(oracle, gpu):
         assert dr.node_struct(nodes[4]).drLastKernelMs == 0.0 and dr.node_struct(nodes[3]).drLastKernelMs > 0.0
 
 
+def test_maxpool_taken_on_load_by_the_1x1_layer_behind_it(oracle, gpu):
+    """SqueezeNet's pool3 / pool5 pattern: fire module -> 3x3/2 max pool -> squeeze 1x1.  With only the last
+    tensor requested the squeeze layer pools while it loads (no pooling launch, no pooled tensor); with
+    DR_FUSE_POOLIN=0 the two kernels run.  Same values to rounding (the channel sum is dealt to a different
+    number of waves), and the layer bar against the oracle either way."""
+    spec, feeds, outs = configs.fire_module(seed=21, size=27, cin=24, squeeze=8, expand=16)
+    st = configs._Streams(22)
+    spec.append(configs._maxpool(outs[0], 3, 2)); pool = len(spec) - 1
+    spec.append(configs._conv(st, pool, 1, 32, 12)); sq = len(spec) - 1
+    want = oracle.run_spec(spec, feeds)
+    res = {}
+    for flag in ("1", "0"):
+        os.environ["DR_FUSE_POOLIN"] = flag
+        try:
+            with dr.Environment() as env:
+                g = env.create_graph()
+                nodes = configs.build_graph(g, spec, [sq])
+                dr.prepare(g)
+                for i, a in feeds.items():
+                    configs.feed_chw(nodes[i], a)
+                dr.graph_config(g).profilingGPU = 1
+                assert g.lib.dR_apply(g.ptr)
+                pool_ms = dr.node_struct(nodes[pool]).drLastKernelMs
+                dr.graph_config(g).profilingGPU = 0
+                assert g.lib.dR_apply(g.ptr) and g.lib.dR_apply(g.ptr)       # recorded, then replayed
+                res[flag] = (configs.fetch_chw(g)[0], pool_ms)
+        finally:
+            os.environ.pop("DR_FUSE_POOLIN", None)
+    assert res["1"][1] == 0.0 and res["0"][1] > 0.0, "the pooling node must launch nothing when fused"
+    assert res["1"][0].shape == (12, 14, 14)
+    assert_close(res["1"][0], want[sq], "squeeze behind pool, fused")
+    assert_close(res["0"][0], want[sq], "squeeze behind pool, unfused")
+    assert rel_err(res["1"][0], res["0"][0]) <= 1e-5
+    # the pooled tensor requested as an output: nothing is fused, and it is there
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes = configs.build_graph(g, spec, [pool, sq])
+        dr.prepare(g)
+        for i, a in feeds.items():
+            configs.feed_chw(nodes[i], a)
+        assert g.lib.dR_apply(g.ptr)
+        got_pool, got_sq = configs.fetch_chw(g)
+    assert_close(got_pool, want[pool], "pool as output")
+    assert_close(got_sq, want[sq], "squeeze, pool as output")
+
+
 def test_fc_chain_fused(oracle, gpu):
     """FC -> FC -> softmax: the finishing kernels of the two GEMVs disappear into their consumers
     (3 launches instead of 5) and the probabilities do not change by a bit."""
@@ -277,7 +323,7 @@ def test_config4_squeezenet(oracle, gpu):
     assert abs(float(probs.sum()) - 1) < 1e-4
     # fused-concat production run gives the same final numbers as the all-outputs run (the two fusions
     # that change a summation order switched off)
-    _, _, prod = run_config("squeezenet", env_vars={"DR_FUSE_EXPAND": "0", "DR_FUSE_AVGPOOL": "0"})
+    _, _, prod = run_config("squeezenet", env_vars={"DR_FUSE_EXPAND": "0", "DR_FUSE_AVGPOOL": "0", "DR_FUSE_POOLIN": "0"})
     assert np.array_equal(prod[len(spec) - 1], got[len(spec) - 1])
     # and with the expand pairs of the 8 fire modules fused into single Winograd launches
     _, _, fused = run_config("squeezenet")

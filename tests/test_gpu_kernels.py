@@ -287,6 +287,32 @@ def test_fc(lib, dev, oracle, C, H, W, N, relu):
         first = got
 
 
+@pytest.mark.parametrize("Win,Hin,I,O", [(56, 56, 128, 32), (28, 28, 256, 48), (55, 27, 20, 7), (9, 6, 3, 17), (2, 2, 1, 1), (1, 1, 5, 3)])
+def test_conv1x1_with_pooled_input(lib, dev, oracle, Win, Hin, I, O):
+    """3x3/2 max pooling taken while the 1x1 layer loads its input: the same values as the pooling kernel
+    followed by the 1x1 GEMM (to rounding: the channel sum may be dealt to a different number of waves),
+    and the oracle's pool -> conv1x1 within the layer bar.
+    Signed inputs: windows hanging over the border must see 0.0, not -inf and not the edge sample."""
+    x, w, b = rnd(I, Hin, Win), rnd(I, O, 1, 1, scale=np.sqrt(2.0 / I)), rnd(O, scale=0.01)
+    Wp, Hp = -(-Win // 2), -(-Hin // 2)
+    pooled = oracle.pool(x, (3, 3, 1), (2, 2, 1), 0)
+    assert pooled.shape == (I, Hp, Wp)
+    xd, wd, bd = dev.put(x), dev.put(w), dev.put(b)
+    for relu in (1, 0):
+        want = oracle.conv1x1(pooled, w, b, relu=bool(relu))
+        out = dev.empty(want.size)
+        ok(lib, lib.drhip_conv1x1_pooled3s2_f32(xd, wd, bd, out, Win, Hin, I, O, relu, None))
+        got = dev.get(out, want.shape)
+        assert_close(got, want, "pooled-input 1x1 %dx%dx%d->%d" % (Win, Hin, I, O))
+        # against the two kernels it replaces
+        mid, two = dev.empty(pooled.size), dev.empty(want.size)
+        ok(lib, lib.drhip_pool_f32(xd, mid, None, Win, Hin, I, 3, 3, 1, 2, 2, 1, 0, None))
+        assert np.array_equal(dev.get(mid, pooled.shape), pooled)
+        ok(lib, lib.drhip_conv1x1_f32(mid, wd, bd, two, Wp * Hp, I, O, relu, 0, None))
+        assert_close(got, dev.get(two, want.shape), "pooled-input 1x1 vs pool + 1x1 kernels")
+    assert lib.drhip_conv1x1_pooled3s2_f32(xd, wd, bd, None, Win, Hin, I, O, 0, None) == -1
+
+
 class DeferredVec(ctypes.Structure):
     """drhip_deferred_vec (include/dr_hip.h)."""
     _fields_ = [("partials", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("slices", ctypes.c_int), ("n", ctypes.c_int), ("relu", ctypes.c_int), ("finished", ctypes.c_void_p),

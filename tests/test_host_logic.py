@@ -328,6 +328,13 @@ def test_schedule_order_and_buffer_plan(lib, oracle, name):
     for i, ins in inputs.items():
         for j in ins:
             last_use[j] = max(last_use[j], pos[i])
+    # a 1x1 layer behind a 3x3/2 max pool that nobody else reads pools while it loads: it reads the tensor
+    # in FRONT of the pooling node, which therefore has to stay intact until that layer has run
+    for i, n in enumerate(spec):
+        if n["op"] == "conv" and tuple(n["w"].shape[2:]) == (1, 1) and spec[n["in"]]["op"] == "pool":
+            pl = spec[n["in"]]
+            if tuple(pl["window"]) == (3, 3, 1) and tuple(pl["stride"]) == (2, 2, 1) and pl["kind"] == 0:
+                last_use[pl["in"]] = max(last_use[pl["in"]], pos[i])
     fused_into = {}
     # a max pool stored by the convolution in front of it: the convolution then owns no tensor of
     # its own, only the pooled one in the pooling node's buffer
