@@ -74,7 +74,7 @@ class GraphStruct(Structure):
                 ("scheduledLayers", c_void_p), ("allNodes", c_void_p), ("debugLayer", c_int),
                 ("drViewHandlers", c_void_p), ("drLastApplyMs", ctypes.c_double), ("drGraphExec", c_void_p),
                 ("drGraphOff", c_int), ("drSideStreams", c_void_p * 3), ("drBranchEvents", c_void_p * 4),
-                ("drBranchGroups", c_int)]
+                ("drBranchGroups", c_int), ("drStaging", c_void_p)]
 
 
 def graph_struct(graph):
@@ -179,6 +179,12 @@ def load_library(path=None):
         "drhip_fc_f32": (c_int, [vp] * 5 + [c_int] * 3 + [vp]),
         "drhip_fc_noalloc_f32": (c_int, [vp] * 4 + [c_int] * 3 + [vp]),
         "drhip_fc_noalloc_max_scratch_floats": (c_size_t, []),
+        "drhip_staging_create": (c_int, [POINTER(vp), c_size_t]),
+        "drhip_staging_destroy": (c_int, [vp]),
+        "drhip_staging_upload_capacity": (c_size_t, [vp]),
+        "drhip_staging_download_capacity": (c_size_t, [vp]),
+        "drhip_upload_staged": (c_int, [vp, vp, c_size_t, vp, c_size_t, vp]),
+        "drhip_download_staged": (c_int, [vp, vp, vp, c_size_t, c_size_t, vp]),
         "drhip_fc_permute_rows_f32": (c_int, [vp, vp] + [c_int] * 4 + [vp]),
         "drhip_softmax_f32": (c_int, [vp, vp, c_int, vp]),
         "drhip_copy3d_f32": (c_int, [vp] + [c_int] * 5 + [vp] + [c_int] * 8 + [vp]),

@@ -24,6 +24,11 @@ __global__ void fill_f32_kernel(float* __restrict__ dst, float value, size_t n) 
     for (; i < n; i += stride) dst[i] = value;
 }
 
+__global__ void copy_f32_kernel(float* __restrict__ dst, const float* __restrict__ src, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
 }  // namespace drhip
 
 using namespace drhip;
@@ -172,6 +177,84 @@ int drhip_download(void* dst, const void* src, size_t off, size_t bytes, void* s
     if (bytes == 0) return DRHIP_OK;
     if (int rc = check(hipMemcpyAsync(dst, (const char*)src + off, bytes, hipMemcpyDeviceToHost, as_stream(stream)), "hipMemcpyAsync(D2H)")) return rc;
     return check(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize(D2H)");
+}
+
+// ---- staged transfers: pinned host memory owned by the library between the caller's pageable arrays and the device
+struct Staging {
+    char* up = nullptr;         // upload area, `cap` bytes
+    char* down = nullptr;       // download area, kStagingDownBytes
+    size_t cap = 0;
+    hipEvent_t upDone = nullptr;
+    bool upPending = false;
+};
+constexpr size_t kStagingDownBytes = 64 * 1024;
+
+int drhip_staging_create(void** handle, size_t upload_bytes) {
+    DRHIP_REQUIRE(handle && upload_bytes > 0, "drhip_staging_create: NULL handle or zero size");
+    Staging* s = new Staging();
+    s->cap = upload_bytes;
+    hipError_t e = hipHostMalloc((void**)&s->up, upload_bytes, hipHostMallocDefault);
+    if (e == hipSuccess) e = hipHostMalloc((void**)&s->down, kStagingDownBytes, hipHostMallocDefault);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&s->upDone, hipEventDisableTiming);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        if (s->up) (void)hipHostFree(s->up);
+        if (s->down) (void)hipHostFree(s->down);
+        delete s;
+        return fail(DRHIP_EDEVICE, "drhip_staging_create: %s", hipGetErrorString(e));
+    }
+    *handle = s;
+    return DRHIP_OK;
+}
+
+int drhip_staging_destroy(void* handle) {
+    Staging* s = (Staging*)handle;
+    if (!s) return DRHIP_OK;
+    if (s->upPending) (void)hipEventSynchronize(s->upDone);
+    (void)hipEventDestroy(s->upDone);
+    (void)hipHostFree(s->up);
+    (void)hipHostFree(s->down);
+    delete s;
+    return DRHIP_OK;
+}
+
+size_t drhip_staging_upload_capacity(void* handle) { return handle ? ((Staging*)handle)->cap : 0; }
+size_t drhip_staging_download_capacity(void* handle) { return handle ? kStagingDownBytes : 0; }
+
+int drhip_upload_staged(void* handle, void* dst, size_t off, const void* src, size_t bytes, void* stream) {
+    Staging* s = (Staging*)handle;
+    DRHIP_REQUIRE(s && dst && src, "drhip_upload_staged: NULL pointer");
+    DRHIP_REQUIRE(bytes <= s->cap, "drhip_upload_staged: %zu bytes do not fit the staging area of %zu", bytes, s->cap);
+    if (bytes == 0) return DRHIP_OK;
+    if (s->upPending) {         // the previous upload may still be reading the area
+        if (int rc = check(hipEventSynchronize(s->upDone), "hipEventSynchronize(staging)")) return rc;
+        s->upPending = false;
+    }
+    // One piece: splitting the array so that the host copy of one piece overlaps the transfer of the one before
+    // was measured slower (0.414 vs 0.386 ms per VGG16 image with 128 KiB pieces: every transfer call costs the
+    // host more than the overlap returns).
+    memcpy(s->up, src, bytes);
+    if (int rc = check(hipMemcpyAsync((char*)dst + off, s->up, bytes, hipMemcpyHostToDevice, as_stream(stream)), "hipMemcpyAsync(H2D, staged)")) return rc;
+    if (int rc = check(hipEventRecord(s->upDone, as_stream(stream)), "hipEventRecord(staging)")) return rc;
+    s->upPending = true;
+    return DRHIP_OK;
+}
+
+int drhip_download_staged(void* handle, void* dst, const void* src, size_t off, size_t bytes, void* stream) {
+    Staging* s = (Staging*)handle;
+    DRHIP_REQUIRE(s && dst && src, "drhip_download_staged: NULL pointer");
+    DRHIP_REQUIRE(bytes <= kStagingDownBytes, "drhip_download_staged: %zu bytes do not fit the staging area of %zu", bytes, kStagingDownBytes);
+    if (bytes == 0) return DRHIP_OK;
+    // A few KiB: a copy kernel that stores straight into the pinned area (it is mapped into the device's address
+    // space) instead of a transfer by the DMA engine, whose start-up costs more than the whole copy.
+    if (((size_t)((const char*)src + off) | bytes) % 4 == 0) {
+        const size_t n = bytes / 4;
+        launch(copy_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, as_stream(stream), (float*)s->down, (const float*)((const char*)src + off), n);
+        if (int rc = launched("copy_f32_kernel")) return rc;
+    } else if (int rc = check(hipMemcpyAsync(s->down, (const char*)src + off, bytes, hipMemcpyDeviceToHost, as_stream(stream)), "hipMemcpyAsync(D2H, staged)")) return rc;
+    if (int rc = check(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize(D2H, staged)")) return rc;
+    memcpy(dst, s->down, bytes);
+    return DRHIP_OK;
 }
 
 int drhip_fill_f32(float* dst, float value, size_t n, void* stream) {

@@ -4,6 +4,7 @@
 // buffer helpers of src/dR_clwrap.c; everything underneath is HIP.
 #include "dr_internal.hpp"
 
+#include <algorithm>
 #include <chrono>
 #include <vector>
 
@@ -192,6 +193,16 @@ gboolean dR_prepare(dR_Graph* net) {
     if (device_failed(net, drhip_stream_sync(stream_of(net)), "dR_prepare(sync)")) return FALSE;
     if (talk) say("Done.\n\n");
 
+    // pinned staging for the per-image copies, sized for the largest feed node (DR_STAGING=0: plain blocking copies)
+    const char* stagingEnv = getenv("DR_STAGING");
+    if (!net->drStaging && !(stagingEnv && strcmp(stagingEnv, "0") == 0)) {
+        size_t largest = 0;
+        for (dR_Node* f : nodes_of(net->feed_layers))
+            largest = std::max(largest, (size_t)f->oshape.s0 * f->oshape.s1 * f->oshape.s2 * sizeof(float));
+        if (largest > 0 && largest <= ((size_t)64 << 20) && drhip_staging_create(&net->drStaging, largest) != DRHIP_OK)
+            net->drStaging = NULL;      // not fatal: the blocking copies still work
+    }
+
     net->prepared = TRUE;
     if (net->config->profilingGPU) {
         say("\nGPU Profiling: Whole graph GPU memory consumption: %4.6f MB \n\n",
@@ -217,8 +228,16 @@ void dR_feedData(dR_Graph* net, dR_Node* feednode, gfloat* data, gint offset, gi
         say("dR_feedData: feed node has no buffer yet (call dR_prepare first) or bad range\n");
         return;
     }
-    dR_uploadArray(net, (gchar*)"", data, (size_t)offset * sizeof(float), (size_t)numfloats * sizeof(float),
-                   feednode->outputBuf->buf);
+    // Per-image path: through the graph's pinned staging area, without waiting for the bus.  The caller's
+    // array has been read when this returns (as with the reference's blocking write, src/deepRACIN.c:76);
+    // the transfer itself is ordered on the graph's stream before the next dR_apply.
+    const size_t bytes = (size_t)numfloats * sizeof(float);
+    if (net->drStaging && data && bytes <= drhip_staging_upload_capacity(net->drStaging)) {
+        device_failed(net, drhip_upload_staged(net->drStaging, (void*)feednode->outputBuf->buf, (size_t)offset * sizeof(float), data, bytes,
+                                               stream_of(net)), "dR_feedData");
+        return;
+    }
+    dR_uploadArray(net, (gchar*)"", data, (size_t)offset * sizeof(float), bytes, feednode->outputBuf->buf);
 }
 
 // One forward pass: walks the schedule and lets every node enqueue its kernels.  Asynchronous
@@ -327,6 +346,7 @@ void dR_cleanup(dR_Graph* net, gboolean cleanupcl) {
     if (talk) say("Cleaning up deepRACIN...\n");
     if (net->clConfig->clContext) drhip_stream_sync(net->clConfig->hipStream);
     if (net->drGraphExec) { drhip_graph_destroy(net->drGraphExec); net->drGraphExec = NULL; }
+    if (net->drStaging) { drhip_staging_destroy(net->drStaging); net->drStaging = NULL; }
     for (int k = 0; k < 4; ++k) { drhip_event_destroy(net->drBranchEvents[k]); net->drBranchEvents[k] = NULL; }
     for (int k = 0; k < 3; ++k) { drhip_stream_destroy(net->drSideStreams[k]); net->drSideStreams[k] = NULL; }
     if (net->prepared) dR_cleanupBuffers(net);
@@ -420,6 +440,11 @@ gboolean dR_uploadArray(dR_Graph* net, gchar*, void* srcHostMem, size_t offset, 
 void dR_downloadArray(dR_Graph* net, gchar*, cl_mem* srcDeviceMem, size_t byteOffset, size_t numBytes,
                       void* destHostMem) {
     if (!srcDeviceMem || !*srcDeviceMem || !destHostMem) { say("dR_downloadArray: NULL buffer\n"); return; }
+    if (net->drStaging && numBytes <= drhip_staging_download_capacity(net->drStaging)) {
+        device_failed(net, drhip_download_staged(net->drStaging, destHostMem, (const void*)*srcDeviceMem, byteOffset, numBytes, stream_of(net)),
+                      "dR_downloadArray");
+        return;
+    }
     device_failed(net, drhip_download(destHostMem, (const void*)*srcDeviceMem, byteOffset, numBytes, stream_of(net)),
                   "dR_downloadArray");
 }

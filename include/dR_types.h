@@ -184,6 +184,7 @@ struct dR_Graph {
     void*           drSideStreams[3];       /* streams that carry independent sibling nodes inside the captured graph */
     void*           drBranchEvents[4];      /* fork event [0] and join events [1..3] of a sibling group */
     gint            drBranchGroups;         /* number of sibling groups the captured graph runs concurrently */
+    void*           drStaging;              /* pinned staging areas for dR_feedData / dR_downloadArray (drhip_staging_create), made by dR_prepare */
 };
 
 struct dR_MemoryHandler {

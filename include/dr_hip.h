@@ -85,6 +85,22 @@ int drhip_free(void* dptr);
 int drhip_upload(void* dst_dev, size_t dst_byte_offset, const void* src_host, size_t bytes, void* stream);
 int drhip_download(void* dst_host, const void* src_dev, size_t src_byte_offset, size_t bytes, void* stream);
 int drhip_fill_f32(float* dst, float value, size_t n, void* stream);
+/* Staged transfers for the per-image copies of a serving loop (the feed of dR_feedData, the logits of
+ * dR_downloadArray).  A staging object owns pinned host memory (hipHostMalloc): an upload area of
+ * `upload_bytes` and a 64 KiB download area.  drhip_upload_staged copies the caller's (pageable) array
+ * into the upload area and starts one transfer from there; it returns when the caller's array has been
+ * read (the array may be reused), NOT when the data is on the device: the transfer is ordered on
+ * `stream` before whatever is enqueued next, and a following staged upload waits for it.
+ * drhip_download_staged blocks like drhip_download; the data comes through the download area, stored
+ * there by a small copy kernel (the area is mapped into the device's address space).  One staging
+ * object serves one stream at a time.  Replace the blocking clEnqueueWriteBuffer / clEnqueueReadBuffer
+ * of dR_uploadArray / dR_downloadArray (src/dR_clwrap.c:1079-1190) on the per-image path. */
+int    drhip_staging_create(void** handle, size_t upload_bytes);
+int    drhip_staging_destroy(void* handle);
+size_t drhip_staging_upload_capacity(void* handle);
+size_t drhip_staging_download_capacity(void* handle);
+int    drhip_upload_staged(void* handle, void* dst_dev, size_t dst_byte_offset, const void* src_host, size_t bytes, void* stream);
+int    drhip_download_staged(void* handle, void* dst_host, const void* src_dev, size_t src_byte_offset, size_t bytes, void* stream);
 
 /* ---- convolution ------------------------------------------------------------------------------
  * Common meaning: in [I][H][W]; out [O][Ho][Wo] with Wo = W/strideX, Ho = H/strideY (floor);

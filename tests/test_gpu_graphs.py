@@ -384,6 +384,49 @@ def test_python_frontend_hwc_roundtrip(oracle, gpu):
     assert rel_err(out, want.transpose(1, 2, 0)) <= LAYER_TOL
 
 
+def test_feed_and_download_through_pinned_staging(oracle, gpu):
+    """dR_feedData goes through the graph's pinned staging area and does not wait for the bus: the caller's
+    array must have been read when the call returns (it is overwritten right after each call here), feeds
+    with an offset and back-to-back feeds must land where and in the order they were made, and
+    DR_STAGING=0 (plain blocking copies) must give the same bytes."""
+    spec, feeds, outs = configs.CONFIGS["conv3x3"](seed=5)
+    x = feeds[0]
+    want = oracle.run_spec(spec, feeds)[outs[0]]
+    res = {}
+    for flag in ("1", "0"):
+        os.environ["DR_STAGING"] = flag
+        try:
+            with dr.Environment() as env:
+                g = env.create_graph()
+                nodes = configs.build_graph(g, spec, outs)
+                dr.prepare(g)
+                assert bool(dr.graph_struct(g).drStaging) == (flag == "1")
+                lib, feed = g.lib, nodes[0]
+                scratch = np.empty_like(x)
+                fp = scratch.ctypes.data_as(dr.POINTER(dr.c_float))
+                outs_seen = []
+                for rep in range(3):
+                    # garbage first, then the real image in two halves from ONE reused host array
+                    scratch[...] = -1e30
+                    lib.dR_feedData(g.ptr, feed.ptr, fp, 0, x.size)
+                    half = x.size // 2
+                    flat = scratch.reshape(-1)
+                    flat[:half] = x.reshape(-1)[:half] * (rep + 1)
+                    lib.dR_feedData(g.ptr, feed.ptr, fp, 0, half)
+                    flat[:x.size - half] = x.reshape(-1)[half:] * (rep + 1)          # overwrites what was just fed
+                    lib.dR_feedData(g.ptr, feed.ptr, fp, half, x.size - half)
+                    scratch[...] = 7e30                                               # and again before the pass runs
+                    assert lib.dR_apply(g.ptr)
+                    outs_seen.append(configs.fetch_chw(g)[0])
+                res[flag] = outs_seen
+        finally:
+            os.environ.pop("DR_STAGING", None)
+    for rep in range(3):
+        assert np.array_equal(res["1"][rep], res["0"][rep])
+    assert_close(res["1"][0], want, "pass fed through the staging area")
+    assert not np.array_equal(res["1"][0], res["1"][1])              # the scaled images really arrived
+
+
 def test_linearity_at_full_size(gpu):
     """Size-independent property at VGG scale: a bias-free linear conv commutes with scaling and adds."""
     rng = np.random.default_rng(5)
