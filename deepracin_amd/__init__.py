@@ -173,6 +173,10 @@ def load_library(path=None):
         "drhip_conv3x3_winograd_pick_variant": (c_int, [c_int] * 4),
         "drhip_conv1x1_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 5 + [vp]),
         "drhip_conv1x1_pick_variant": (c_int, [c_int] * 3),
+        "drhip_conv3x3_direct_filter_floats": (c_size_t, [c_int, c_int]),
+        "drhip_conv3x3_direct_filter_layout_f32": (c_int, [vp, vp, c_int, c_int, vp]),
+        "drhip_conv3x3_direct_pick_variant": (c_int, [c_int] * 4),
+        "drhip_conv3x3_direct_mfma_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 7 + [vp]),
         "drhip_conv1x1_pooled3s2_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 5 + [vp]),
         "drhip_pool_f32": (c_int, [vp, vp, vp] + [c_int] * 10 + [vp]),
         "drhip_fc_scratch_floats": (c_size_t, [c_int, c_int]),

@@ -19,6 +19,7 @@
 #include <cfloat>
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 namespace drhip {
 
@@ -358,146 +359,187 @@ conv3x3_fewc_mfma_kernel(const float* __restrict__ in, const float* __restrict__
 }
 
 // Direct 3x3 convolution on the matrix cores (stride 1 or 2, more than 4 input channels): the
-// implicit GEMM  out[o][p] = sum_{c,tap} w[c][o][tap] * in[c][pixel p shifted by tap],  K = 9*I.
+// implicit GEMM  out[o][p] = sum_{c,tap} w[c][o][tap] * in[c][pixel p shifted by tap],  K = 9*I,
+// on v_mfma_f32_32x32x2_f32, with no operand staged in LDS:
 //
-// A workgroup (4 waves) owns 32 output channels x NY MFMA column groups of 32 output pixels (a
-// 16 x 2*NY block; NY = 2 for layers large enough to fill the chip that way: a staged filter then
-// feeds two MFMAs) and walks the input channels 16 at a time.  A stage's zero-padded input patch and
-// its filters (re-laid [c][tap][o]) are staged in LDS by all lanes, double buffered: the global
-// loads of stage s+1 are in flight while stage s is multiplied.  Inside a stage the four waves
-// split the channels (4 each = two k-steps of v_mfma_f32_32x32x2_f32 per tap, 18 MFMAs), every
-// operand is one ds_read_b32; the four partial tiles meet in LDS at the end (wave order, so the
-// summation order is fixed), then bias, ReLU and 64-byte row stores.  Small layers get enough
-// workgroups from the small pixel block (56x56 -> 64 channels: 224), large ones are MFMA-bound.
-constexpr int kDmTX = 16;                   // output block: 16 x 2*NY pixels
-constexpr int kDmCC = 16;                   // input channels per stage
-constexpr int kDmThreads = 256;
+//   * the filters are laid out once, at prepare time, as F[tap][c/8][o][8] -- the layout of the Winograd
+//     kernel's transformed filters with 9 taps in place of 16 transform positions: inside a chunk of 8
+//     channels channel c%8 sits at position (c&1)*4 + (c%8)/2, so the A operands of the four k-steps of a
+//     stage (k-step ks needs channel 2ks + lane/32) are ONE aligned 16-byte buffer load per lane and tap;
+//   * the B operands are the input itself: a lane owns one output pixel (lane%32) and one channel parity
+//     (lane/32) and loads the three rows of its 3x3 window with one 16-byte buffer load each (rows outside
+//     the image carry an offset beyond the resource and read 0.0; the samples left and right of the image
+//     are zeroed by selects).  Neighbouring lanes load overlapping windows; the CU's L1 absorbs that.
+//   * a workgroup owns 32 consecutive output pixels (row-major) x 32*NT output channels; its KW waves deal
+//     the 8-channel stages round-robin (wave w takes stages w, w+KW, ...), the next stage's rows in flight
+//     during the 36*NT MFMAs of the current one and the filters of a tap reloaded right behind its MFMAs;
+//     the KW partial tiles meet in LDS at the end and are added in wave order (fixed summation order),
+//     then bias, ReLU and 128-byte row stores.
+// Per stage and wave: 12 + 9*NT loads and ~50 VALU instructions (the selects) for 36*NT MFMAs.
+typedef float f32x16d __attribute__((ext_vector_type(16)));
+typedef float f32x4d __attribute__((ext_vector_type(4)));
+constexpr unsigned kDmBufferFlags = 0x00020000u;    // dword 3 of a gfx9 raw buffer resource (32-bit data format)
+constexpr unsigned kDmOutOfRange = 0x80000000u;     // byte offset no resource of at most 2 GiB contains
+constexpr int kDmKC = 8;                            // input channels per stage (4 MFMA k-steps)
 constexpr int kDmPartPitch = 33;
 
-template <int S, int NY>                    // stride (both directions): 1 or 2; column groups per wave
-__global__ void __launch_bounds__(kDmThreads)
-conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
-                           float* __restrict__ out, int W, int H, int I, int O, int Wo, int Ho, int tilesX, int relu) {
-    constexpr int kDmTY = 2 * NY;
-    constexpr int PH = (kDmTY - 1) * S + 3, PW = (kDmTX - 1) * S + 3;      // input patch of the block
-    constexpr int kPatch = kDmCC * PH * PW, kFilt = kDmCC * 9 * 32;         // floats per stage
-    constexpr int kPatchLoads = (kPatch + kDmThreads - 1) / kDmThreads;
-    constexpr int kFiltLoads = (kFilt / 4 + kDmThreads - 1) / kDmThreads;   // 16-byte loads
-    extern __shared__ float lds[];              // [2][kPatch + kFilt]; reused for the partial tiles at the end
-    typedef float f32x16d __attribute__((ext_vector_type(16)));
-    typedef float f32x4l __attribute__((ext_vector_type(4)));
+__host__ __device__ inline int dm_opad(int O) { return (O + 31) / 32 * 32; }
+__host__ __device__ inline size_t dm_filter_index(int tap, int c, int o, int nChunks, int Opad) {
+    const int cc = c & 7;
+    return (((size_t)tap * nChunks + (c >> 3)) * Opad + o) * 8 + (cc & 1) * 4 + (cc >> 1);
+}
+
+// F[tap][c/8][o][8] from w[c][o][3][3]; channels >= I and output channels >= O (padded to a multiple of 32) are zero.
+__global__ void __launch_bounds__(256)
+direct_filter_layout_kernel(const float* __restrict__ w, float* __restrict__ F, int I, int O, int nChunks) {
+    const int Opad = dm_opad(O);
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= nChunks * 8 * Opad) return;
+    const int c = idx / Opad, o = idx % Opad;
+    const bool real = c < I && o < O;
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) F[dm_filter_index(tap, c, o, nChunks, Opad)] = real ? w[((size_t)c * O + o) * 9 + tap] : 0.0f;
+}
+
+__device__ inline f32x4d dm_buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset) {
+    return __builtin_bit_cast(f32x4d, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voffset, (int)soffset, 0));
+}
+
+template <int NT, int S>                    // 32*NT output channels per workgroup; stride (both directions) 1 or 2
+__global__ void __launch_bounds__(512)
+conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict__ F, const float* __restrict__ bias,
+                           float* __restrict__ out, int W, int H, int I, int O, int Wo, int Ho, int nPT, int relu) {
+    constexpr int OB = 32 * NT, KC = kDmKC;
+    constexpr int NA = NT == 1 ? 2 : 1;     // accumulators per channel block: two independent MFMA chains at least
+    extern __shared__ float part[];         // [KW][OB][kDmPartPitch]
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int j = lane & 31, kpar = lane >> 5;
-    const int xx = j & 15, yy = j >> 4;
-    const int tileX = blockIdx.x % tilesX, tileY = blockIdx.x / tilesX;
-    const int o0 = blockIdx.y * 32;
-    const int x0 = tileX * kDmTX, y0 = tileY * kDmTY;
-    const int ix0 = x0 * S - 1, iy0 = y0 * S - 1;
-    const int nStages = (I + kDmCC - 1) / kDmCC;
-    const bool wholeTile = o0 + 32 <= O;        // the 16-byte filter loads need all 32 channels to exist
+    const int KW = blockDim.x >> 6;
+    const int l32 = lane & 31, lhi = lane >> 5;
+    const int o0 = (blockIdx.x / nPT) * OB, p0 = (blockIdx.x % nPT) * 32;
+    const int P = Wo * Ho, plane = H * W;
+    const int nChunks = (I + KC - 1) / KC, Opad = dm_opad(O);
 
-    float pv[kPatchLoads];
-    f32x4l fv[kFiltLoads];
-    auto load_stage = [&](int s) {
-        const int c0 = s * kDmCC;
+    // this lane's output pixel and the byte offsets of its three window rows
+    const int p = p0 + l32;
+    const bool pOk = p < P;
+    const int pc = min(p, P - 1);
+    const int y = pc / Wo, x = pc - y * Wo;
+    // The window starts at column x*S - 1.  Only x = 0 starts left of the image: that lane loads from column 0
+    // and shifts its samples up by one (a negative offset would zero the whole load for the first pixel).
+    const bool shifted = x == 0;
+    const int xLoad = x * S - 1 + (shifted ? 1 : 0);
+    const bool c2ok = x * S + 1 < W;        // the third sample of the window exists
+    unsigned offRow[3];
 #pragma unroll
-        for (int u = 0; u < kPatchLoads; ++u) {
-            const int e = tid + u * kDmThreads;
-            const int c = min(e / (PH * PW), kDmCC - 1), rem = e % (PH * PW);
-            const int gy = iy0 + rem / PW, gx = ix0 + rem % PW;
-            const bool ok = e < kPatch && c0 + c < I && gy >= 0 && gy < H && gx >= 0 && gx < W;
-            const float v = in[((size_t)min(c0 + c, I - 1) * H + min(max(gy, 0), H - 1)) * W + min(max(gx, 0), W - 1)];
-            pv[u] = ok ? v : 0.0f;
-        }
-#pragma unroll
-        for (int u = 0; u < kFiltLoads; ++u) {
-            const int f = 4 * (tid + u * kDmThreads);                       // first of four floats in [c][o][tap] order
-            const int c = min(f / 288, kDmCC - 1), rem = f % 288;
-            if (wholeTile && c0 + kDmCC <= I) {                             // workgroup-uniform
-                fv[u] = *(const f32x4l*)(w + ((size_t)(c0 + c) * O + o0) * 9 + rem);
-            } else {
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int ol = (rem + k) / 9, tap = (rem + k) % 9;
-                    const float v = w[((size_t)min(c0 + c, I - 1) * O + min(o0 + ol, O - 1)) * 9 + tap];
-                    fv[u][k] = (c0 + c < I && o0 + ol < O) ? v : 0.0f;
-                }
-            }
-        }
-    };
-    auto store_stage = [&](float* buf) {
-        float* patch = buf;
-        float* filt = buf + kPatch;
-#pragma unroll
-        for (int u = 0; u < kPatchLoads; ++u) {
-            const int e = tid + u * kDmThreads;
-            if (e < kPatch) patch[e] = pv[u];
-        }
-#pragma unroll
-        for (int u = 0; u < kFiltLoads; ++u) {
-            const int f = 4 * (tid + u * kDmThreads);
-            if (f < kFilt) {
-                const int c = f / 288, rem = f % 288;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) filt[(c * 9 + (rem + k) % 9) * 32 + (rem + k) / 9] = fv[u][k];
-            }
-        }
-    };
-
-    f32x16d acc[NY];
-#pragma unroll
-    for (int g = 0; g < NY; ++g)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[g][r] = 0.0f;
-
-    load_stage(0);
-    store_stage(lds);
-    __syncthreads();
-    for (int s = 0; s < nStages; ++s) {
-        const float* buf = lds + (s & 1) * (kPatch + kFilt);
-        if (s + 1 < nStages) load_stage(s + 1);
-        const float* patch = buf;
-        const float* filt = buf + kPatch;
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-            const int ch = 4 * wave + 2 * ks + kpar;                        // channel within the stage
-#pragma unroll
-            for (int tap = 0; tap < 9; ++tap) {
-                const float a = filt[(ch * 9 + tap) * 32 + j];
-#pragma unroll
-                for (int g = 0; g < NY; ++g) {
-                    const float b = patch[(ch * PH + (2 * g + yy) * S + tap / 3) * PW + xx * S + tap % 3];
-                    acc[g] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[g], 0, 0, 0);
-                }
-            }
-        }
-        if (s + 1 < nStages) store_stage(lds + ((s + 1) & 1) * (kPatch + kFilt));
-        __syncthreads();
+    for (int d = 0; d < 3; ++d) {
+        const int iy = y * S - 1 + d;
+        offRow[d] = (pOk && iy >= 0 && iy < H) ? 4u * (unsigned)(lhi * plane + iy * W + xLoad) : kDmOutOfRange;
     }
 
-    // partial tiles of the four waves -> LDS -> summed in wave order
-    float* part = lds;
+    const __amdgpu_buffer_rsrc_t rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kDmBufferFlags);
+    const __amdgpu_buffer_rsrc_t rF = __builtin_amdgcn_make_buffer_rsrc((void*)F, 0, 9 * nChunks * Opad * 8 * 4, kDmBufferFlags);
+    const unsigned fOff = 4u * (unsigned)((o0 + l32) * 8 + 4 * lhi);
+
+    // rows of channels cbase + 2ks + lhi, ks = 0..3.  Plain form: one resource for the tensor, the channel in the
+    // scalar offset (chunks known to lie inside the tensor).  Ranged form: the resource starts at channel cbase and
+    // ends with the tensor, so channels >= I read 0.0 (ragged last chunk, prefetch past the end).
+    auto load_rows_plain = [&](f32x4d (&raw)[4][3], int cbase) {
 #pragma unroll
-    for (int g = 0; g < NY; ++g) {
+        for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-            part[(wave * 32 + 8 * (r / 4) + 4 * kpar + (r % 4)) * kDmPartPitch + j] = acc[g][r];
-        __syncthreads();
-        for (int idx = tid; idx < 32 * 32; idx += kDmThreads) {
-            const int ol = idx >> 5, pl = idx & 31;
-            const int o = o0 + ol, x = x0 + (pl & 15), y = y0 + 2 * g + (pl >> 4);
-            float v = 0.0f;
+            for (int d = 0; d < 3; ++d) raw[ks][d] = dm_buf_load4(rIn, offRow[d], 4u * (unsigned)((cbase + 2 * ks) * plane));
+    };
+    auto load_rows_ranged = [&](f32x4d (&raw)[4][3], int cbase) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) v += part[(k * 32 + ol) * kDmPartPitch + pl];
-            if (o < O && x < Wo && y < Ho) {
-                if (bias) v += bias[o];
-                if (relu) v = fmaxf(v, 0.0f);
-                out[((size_t)o * Ho + y) * Wo + x] = v;
-            }
+        for (int ks = 0; ks < 4; ++ks) {
+            const int c = cbase + 2 * ks, left = max(I - c, 0);
+            const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(in + (size_t)min(c, I) * plane), 0, left * plane * 4, kDmBufferFlags);
+#pragma unroll
+            for (int d = 0; d < 3; ++d) raw[ks][d] = dm_buf_load4(r, offRow[d], 0u);
         }
-        if (g + 1 < NY) __syncthreads();        // the partial tiles are overwritten by the next group
+    };
+    auto load_filters = [&](f32x4d (&f)[NT], int tap, int chunk) {
+        const unsigned soff = 4u * (unsigned)((tap * nChunks + chunk) * Opad * 8);
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) f[nt] = dm_buf_load4(rF, fOff + 4u * (unsigned)(nt * 32 * 8), soff);
+    };
+
+    f32x16d acc[NT][NA];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int a = 0; a < NA; ++a)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[nt][a][r] = 0.0f;
+
+    f32x4d raw[4][3];
+    f32x4d f[9][NT];
+    if (wave < nChunks) {
+        load_rows_ranged(raw, wave * KC);
+#pragma unroll
+        for (int tap = 0; tap < 9; ++tap) load_filters(f[tap], tap, wave);
+    }
+
+    auto stage = [&](int ch, auto plainNext) {
+        const int next = min(ch + KW, nChunks - 1);
+        // the window samples of this stage, padding applied: b[ks][3*d + e] = in[c][y*S - 1 + d][x*S - 1 + e]
+        float b[4][9];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int d = 0; d < 3; ++d) {
+                const f32x4d v = raw[ks][d];
+                b[ks][3 * d + 0] = shifted ? 0.0f : v[0];
+                b[ks][3 * d + 1] = shifted ? v[0] : v[1];
+                const float third = shifted ? v[1] : v[2];
+                b[ks][3 * d + 2] = c2ok ? third : 0.0f;
+            }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (decltype(plainNext)::value) load_rows_plain(raw, (ch + KW) * KC);
+        else load_rows_ranged(raw, (ch + KW) * KC);
+#pragma unroll
+        for (int tap = 0; tap < 9; ++tap) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    acc[nt][tap % NA] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[tap][nt][ks], b[ks][tap], acc[nt][tap % NA], 0, 0, 0);
+            load_filters(f[tap], tap, next);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // stages whose successor (KW further on) is a complete chunk prefetch in the plain form
+    const int chMain = I / KC - KW;
+    int ch = wave;
+    for (; ch < chMain; ch += KW) stage(ch, std::true_type{});
+    for (; ch < nChunks; ch += KW) stage(ch, std::false_type{});
+
+    // partial tiles of the KW waves -> LDS -> summed in wave order.  Accumulator layout of the 32x32 MFMA:
+    // lane -> column (pixel) lane%32; register r -> row (channel) 8*(r/4) + 4*(lane/32) + r%4.
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float v = acc[nt][0][r];
+            if constexpr (NA == 2) v += acc[nt][1][r];
+            part[(wave * OB + 32 * nt + 8 * (r / 4) + 4 * lhi + (r % 4)) * kDmPartPitch + l32] = v;
+        }
+    // LDS-only barrier: __syncthreads() would also wait for the outstanding (unused) prefetches
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    for (int idx = tid; idx < OB * 32; idx += blockDim.x) {
+        const int ol = idx >> 5, pl = idx & 31;
+        const int o = o0 + ol, pp = p0 + pl;
+        float v = 0.0f;
+        for (int k = 0; k < KW; ++k) v += part[(k * OB + ol) * kDmPartPitch + pl];
+        if (o < O && pp < P) {
+            if (bias) v += bias[o];
+            if (relu) v = fmaxf(v, 0.0f);
+            out[(size_t)o * P + pp] = v;
+        }
     }
 }
 
@@ -564,24 +606,6 @@ extern "C" int drhip_conv2d_direct_f32(const float* in, const float* w, const fl
 #undef DRHIP_FEWC
         return launched("conv_direct_fewc_kernel");
     }
-    if (kw == 3 && kh == 3 && strideX == strideY && (strideX == 1 || strideX == 2) && !valu) {
-        // matrix-core form: 32 channels x (16 x 2) pixels per workgroup, 16 input channels per stage
-        const int Wo = W / strideX, Ho = H / strideY;
-        // 16 x 4 pixel blocks when those alone give every CU a workgroup, else 16 x 2 (stride 2
-        // always: its double-buffered patch of a 16 x 4 block would not fit 64 KiB of LDS)
-        const int ny = (strideX == 1 && ceil_div(Wo, kDmTX) * ceil_div(Ho, 4) * ceil_div(O, 32) >= num_cu()) ? 2 : 1;
-        const int tilesX = ceil_div(Wo, kDmTX), tilesY = ceil_div(Ho, 2 * ny);
-        const dim3 grid(tilesX * tilesY, ceil_div(O, 32)), block(kDmThreads);
-        const int PH = (2 * ny - 1) * strideX + 3, PW = (kDmTX - 1) * strideX + 3;
-        const size_t stage = (size_t)kDmCC * PH * PW + (size_t)kDmCC * 9 * 32;
-        const size_t ldsFloats = 2 * stage > (size_t)4 * 32 * kDmPartPitch ? 2 * stage : (size_t)4 * 32 * kDmPartPitch;
-        DRHIP_REQUIRE(ldsFloats * sizeof(float) <= 64 * 1024, "drhip_conv2d_direct_f32: internal: LDS stage too large");
-#define DRHIP_DM(SV, NYV) launch((conv3x3_direct_mfma_kernel<SV, NYV>), grid, block, ldsFloats * sizeof(float), s0, in, w, bias, out, W, H, I, O, Wo, Ho, tilesX, relu)
-        if (strideX == 1) { if (ny == 2) DRHIP_DM(1, 2); else DRHIP_DM(1, 1); }
-        else DRHIP_DM(2, 1);
-#undef DRHIP_DM
-        return launched("conv3x3_direct_mfma_kernel");
-    }
     // Few output channels per lane when the tile count alone cannot fill the CUs.
     const int tiles = ceil_div(W / strideX, kDirTile) * ceil_div(H / strideY, kDirTile);
     hipStream_t s = as_stream(stream);
@@ -610,4 +634,58 @@ extern "C" int drhip_conv3x3_pool3s2_f32(const float* in, const float* w, const 
 #undef DRHIP_FP_K
 #undef DRHIP_FP
     return launched("conv3x3_fewc_pool3s2_kernel");
+}
+
+extern "C" size_t drhip_conv3x3_direct_filter_floats(int I, int O) {
+    if (I <= 0 || O <= 0) return 0;
+    return (size_t)9 * ceil_div(I, kDmKC) * kDmKC * dm_opad(O);
+}
+
+extern "C" int drhip_conv3x3_direct_filter_layout_f32(const float* w, float* F, int I, int O, void* stream) {
+    DRHIP_REQUIRE(w && F, "drhip_conv3x3_direct_filter_layout_f32: NULL tensor");
+    DRHIP_REQUIRE(I > 0 && O > 0 && (long long)(I + 7) * (O + 31) * 9 < (1ll << 29), "drhip_conv3x3_direct_filter_layout_f32: bad shape I=%d O=%d", I, O);
+    const int nChunks = ceil_div(I, kDmKC);
+    launch(direct_filter_layout_kernel, dim3(ceil_div(nChunks * 8 * dm_opad(O), 256)), dim3(256), 0, as_stream(stream), w, F, I, O, nChunks);
+    return launched("direct_filter_layout_kernel");
+}
+
+// variant = waves per workgroup (1, 2, 4, 8) | 0x10 for 64 output channels per workgroup (else 32)
+extern "C" int drhip_conv3x3_direct_pick_variant(int Wo, int Ho, int I, int O) {
+    const int nChunks = ceil_div(I, kDmKC);
+    const int tiles = ceil_div(Wo * Ho, 32);
+    // 64 channels per workgroup share every window between two MFMA sets; taken once such blocks alone give every
+    // CU a workgroup (56x56, 256 -> 256: 44.1 us against 46.8 us with 32-channel blocks)
+    const bool wide = O >= 64 && tiles * ceil_div(O, 64) >= num_cu();
+    // four waves per workgroup, fewer when that would leave a wave less than two stages; eight for layers with
+    // fewer workgroups than CUs (56x56, 64 -> 64: 6.5 us against 7.4 us)
+    int kw = 1;
+    while (kw < 4 && nChunks >= 4 * kw) kw *= 2;
+    if (tiles * ceil_div(O, wide ? 64 : 32) < num_cu() && nChunks >= 8) kw = 8;
+    return kw | (wide ? 0x10 : 0);
+}
+
+extern "C" int drhip_conv3x3_direct_mfma_f32(const float* in, const float* F, const float* bias, float* out,
+                                             int W, int H, int I, int O, int stride, int relu, int variant, void* stream) {
+    DRHIP_REQUIRE(in && F && out, "drhip_conv3x3_direct_mfma_f32: NULL tensor");
+    DRHIP_REQUIRE(W > 0 && H > 0 && I > 0 && O > 0, "drhip_conv3x3_direct_mfma_f32: bad shape %dx%dx%d -> %d", W, H, I, O);
+    DRHIP_REQUIRE(stride == 1 || stride == 2, "drhip_conv3x3_direct_mfma_f32: stride %d (1 or 2)", stride);
+    const int Wo = W / stride, Ho = H / stride;
+    DRHIP_REQUIRE(Wo > 0 && Ho > 0, "drhip_conv3x3_direct_mfma_f32: output is empty");
+    // byte offsets into the input and the filters are 32-bit, and 0x80000000 must lie outside both
+    DRHIP_REQUIRE((long long)W * H * I < (1ll << 29) && (long long)Wo * Ho * O < (1ll << 31) && (long long)(I + 7) * (O + 31) * 9 < (1ll << 29),
+                  "drhip_conv3x3_direct_mfma_f32: tensor too large for 32-bit byte offsets");
+    DRHIP_REQUIRE(((size_t)F & 15) == 0, "drhip_conv3x3_direct_mfma_f32: the filter bank must be 16-byte aligned");
+    if (variant == 0) variant = drhip_conv3x3_direct_pick_variant(Wo, Ho, I, O);
+    const int kw = variant & 0xf, wide = (variant & 0x10) != 0;
+    DRHIP_REQUIRE((variant >> 5) == 0 && (kw == 1 || kw == 2 || kw == 4 || kw == 8), "drhip_conv3x3_direct_mfma_f32: unknown variant %#x", variant);
+    const int OB = wide ? 64 : 32;
+    const int nPT = ceil_div(Wo * Ho, 32);
+    const dim3 grid(nPT * ceil_div(O, OB)), block(64 * kw);
+    const size_t ldsBytes = (size_t)kw * OB * kDmPartPitch * sizeof(float);
+    hipStream_t s = as_stream(stream);
+#define DRHIP_DM(NTV, SV) launch((conv3x3_direct_mfma_kernel<NTV, SV>), grid, block, ldsBytes, s, in, F, bias, out, W, H, I, O, Wo, Ho, nPT, relu)
+    if (wide) { if (stride == 1) DRHIP_DM(2, 1); else DRHIP_DM(2, 2); }
+    else { if (stride == 1) DRHIP_DM(1, 1); else DRHIP_DM(1, 2); }
+#undef DRHIP_DM
+    return launched("conv3x3_direct_mfma_kernel");
 }

@@ -76,7 +76,15 @@ gboolean conv_schedule(dR_Graph* net, dR_Node* node) {
     switch (c->algo) {
         case drConvWinograd: c->variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O); break;
         case drConv1x1Gemm:  c->variant = drhip_conv1x1_pick_variant(W * H, I, O); break;
-        default:             c->variant = 0; break;      // the direct launcher sizes its own tiles
+        default: {
+            // 3x3, stride 1 or 2, more than 4 input channels: the implicit GEMM on the matrix cores over a filter
+            // bank laid out at prepare time; everything else: the direct launcher sizes its own tiles
+            const char* valu = getenv("DR_DIRECT_VALU");
+            c->drDirectBank = c->shape.s0 == 3 && c->shape.s1 == 3 && I > 4 && c->stride.s1 == c->stride.s2 &&
+                              (c->stride.s1 == 1 || c->stride.s1 == 2) && !(valu && strcmp(valu, "1") == 0);
+            c->variant = c->drDirectBank ? drhip_conv3x3_direct_pick_variant(W / c->stride.s1, H / c->stride.s2, I, O) : 0;
+            break;
+        }
     }
     if ((c->shape.s0 & 1) == 0 || (c->shape.s1 & 1) == 0) {
         say("Conv2d Layer %d: filter %dx%d must have odd side lengths! \n", node->layerID, c->shape.s0, c->shape.s1);
@@ -107,7 +115,8 @@ gboolean conv_allocate(dR_Graph* net, dR_Node* node) {
     const int O = launch_channels(c);
     if (c->drAbsorbed1x1)                       // the joint layer is wider than the one schedule() saw
         c->variant = drhip_conv3x3_winograd_pick_variant(c->ishape.s0, c->ishape.s1, c->shape.s2, O);
-    const int n = wino ? (int)drhip_conv3x3_winograd_filter_floats(c->shape.s2, O) : weight_count(c);
+    const int n = wino ? (int)drhip_conv3x3_winograd_filter_floats(c->shape.s2, O)
+                       : c->drDirectBank ? (int)drhip_conv3x3_direct_filter_floats(c->shape.s2, O) : weight_count(c);
     gboolean ok = dR_createFloatBuffer(net, &c->weightsBuf, n, CL_MEM_READ_ONLY);
     if (launch_has_bias(c)) ok = ok && dR_createFloatBuffer(net, &c->biasBuf, O, CL_MEM_READ_ONLY);
     const size_t ws = wino ? drhip_conv3x3_winograd_workspace_floats(c->ishape.s0, c->ishape.s1, c->shape.s2, O, c->variant) : 0;
@@ -154,6 +163,18 @@ gboolean conv_fill(dR_Graph* net, dR_Node* node) {
             if (c->useBias) memcpy(bias.data() + O1, c->biases, (size_t)O3 * sizeof(float));
             return dR_uploadArray(net, (gchar*)"", bias.data(), 0, (size_t)O * sizeof(float), c->biasBuf);
         }
+    } else if (c->drDirectBank) {
+        // raw weights go up once, the filter bank is laid out on the device, the raw copy is dropped
+        const int I = c->shape.s2, O = c->shape.s3;
+        const size_t rawBytes = (size_t)weight_count(c) * sizeof(float);
+        cl_mem raw = NULL;
+        if (!dR_createFloatBuffer(net, &raw, weight_count(c), CL_MEM_READ_ONLY)) return FALSE;
+        ok = dR_uploadArray(net, (gchar*)"", c->weights, 0, rawBytes, raw);
+        if (ok) ok = !device_failed(net, drhip_conv3x3_direct_filter_layout_f32((const float*)raw, (float*)c->weightsBuf, I, O, stream_of(net)),
+                                    "direct filter layout");
+        if (ok) ok = !device_failed(net, drhip_stream_sync(stream_of(net)), "direct filter layout (sync)");
+        dR_clMemoryBufferCleanup(net, raw);
+        net->clConfig->memConsumptionGPU -= (glong)rawBytes;
     } else {
         ok = dR_uploadArray(net, (gchar*)"", c->weights, 0, (size_t)weight_count(c) * sizeof(float), c->weightsBuf);
     }
@@ -193,6 +214,8 @@ gboolean conv_compute(dR_Graph* net, dR_Node* node) {
         default:
             if (c->drFusedPool)                 // first layer + the 3x3/2 max pool behind it (out = the pool's buffer)
                 rc = drhip_conv3x3_pool3s2_f32(in, w, b, out, W, H, I, O, c->stride.s1, c->stride.s2, relu, stream_of(net));
+            else if (c->drDirectBank)
+                rc = drhip_conv3x3_direct_mfma_f32(in, w, b, out, W, H, I, O, c->stride.s1, relu, c->variant, stream_of(net));
             else
                 rc = drhip_conv2d_direct_f32(in, w, b, out, W, H, I, O, c->shape.s0, c->shape.s1,
                                              c->stride.s1, c->stride.s2, relu, stream_of(net));

@@ -51,6 +51,8 @@ struct dR_Conv2d_Data {
                                            in workspaceBuf and neither its tensor nor the pooled one is computed by a kernel of its own */
     gboolean            drFusedPool;    /* set by the buffer planner: the node's only consumer is a 2x2/2 max pool and
                                            this node writes the pooled tensor straight into that node's buffer */
+    gboolean            drDirectBank;   /* set by schedule() on a direct 3x3 layer with more than 4 input channels and stride
+                                           1 or 2: weightsBuf holds the filter bank of the matrix-core kernel, variant its tiles */
     dR_Node*            drPooledInput;  /* set by the buffer planner on a 1x1 layer whose input is a 3x3/2 max pooling
                                            read by nobody else: that pooling node; the layer reads the pooling's own
                                            input and takes the window maxima while loading, the pooling launches nothing */

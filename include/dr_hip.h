@@ -115,6 +115,23 @@ int drhip_conv2d_direct_f32(const float* in, const float* w, const float* bias, 
                             int W, int H, int I, int O, int kw, int kh,
                             int strideX, int strideY, int relu, void* stream);
 
+/* Direct 3x3 convolution (stride 1 or 2 in both directions, zero padding 1) as an implicit GEMM with
+ * K = 9*I on the fp32 MFMA units, for layers with more than 4 input channels.  F is the filter bank in
+ * the layout the kernel streams, produced once at prepare time from w [I][O][3][3]:
+ * F[tap][c/8][o][8], tap = 3*j + i, input channels padded with zeros to a multiple of 8, output
+ * channels to a multiple of 32, and channel c%8 stored at position (c&1)*4 + (c%8)/2 of its group of 8;
+ * drhip_conv3x3_direct_filter_floats(I,O) floats.  `variant` (0 = let the launcher pick) = waves per
+ * workgroup (1, 2, 4, 8: they deal the 8-channel stages round-robin, partial tiles added in wave
+ * order) | 0x10 for 64 instead of 32 output channels per workgroup.  Same function as
+ * drhip_conv2d_direct_f32 with kw = kh = 3.  Replaces the per-layer generated kernel
+ * `conv2d3x3x<O>_<id>_...` and its launch (src/dR_nodes_conv2d.c:364-420, 481-773); the reference
+ * re-lays nothing (it reads [I][O][3][3] through __constant or global memory). */
+size_t drhip_conv3x3_direct_filter_floats(int I, int O);
+int drhip_conv3x3_direct_filter_layout_f32(const float* w /* [I][O][3][3] */, float* F, int I, int O, void* stream);
+int drhip_conv3x3_direct_pick_variant(int Wo, int Ho, int I, int O);
+int drhip_conv3x3_direct_mfma_f32(const float* in, const float* F, const float* bias, float* out,
+                                  int W, int H, int I, int O, int stride, int relu, int variant, void* stream);
+
 /* First layer (1 to 4 input channels, 3x3, any stride, zero padding, bias, optional ReLU) followed by
  * a 3x3 / stride-2 max pooling with the reference's pooling rules (out = ceil(in/2), samples outside
  * the map read 0.0): out[O][ceil(Ho/2)][ceil(Wo/2)], Wo = W/strideX, Ho = H/strideY.  The

@@ -69,7 +69,7 @@ def ok(lib, rc):
     (224, 224, 3, 64, 3, 2),     # SqueezeNet conv1
     (17, 13, 5, 7, 3, 1), (20, 18, 4, 20, 5, 1), (33, 31, 3, 9, 3, 2), (16, 16, 2, 3, 7, 3), (9, 9, 1, 1, 1, 2),
     (37, 21, 4, 33, 3, 1), (8, 5, 1, 16, 3, 3), (2, 2, 3, 2, 3, 1),     # I <= 4 with a 3x3 filter: the no-LDS first-layer kernel
-    (112, 110, 24, 40, 3, 1), (61, 37, 17, 70, 3, 2), (30, 9, 8, 32, 3, 1),   # 3x3 on the matrix cores: 16x4 blocks, stride 2, ragged channels
+    (112, 110, 24, 40, 3, 1), (61, 37, 17, 70, 3, 2), (30, 9, 8, 32, 3, 1),   # 3x3 with raw weights and more than 4 channels: the LDS-tiled kernel
 ])
 def test_conv_direct(lib, dev, oracle, W, H, I, O, k, s):
     x, w, b = np.abs(rnd(I, H, W)), rnd(I, O, k, k, scale=np.sqrt(2.0 / (k * k * I))), rnd(O, scale=0.01)
@@ -82,6 +82,42 @@ def test_conv_direct(lib, dev, oracle, W, H, I, O, k, s):
     want2 = oracle.conv_direct(x, w, None, (s, s), relu=False)
     ok(lib, lib.drhip_conv2d_direct_f32(dev.put(x), dev.put(w), None, out, W, H, I, O, k, k, s, s, 0, None))
     assert_close(dev.get(out, want2.shape), want2)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 4, 8, 0x11, 0x14, 0x18])
+@pytest.mark.parametrize("W,H,I,O,s", [
+    (56, 56, 64, 64, 1),         # config 1, direct variant
+    (56, 56, 128, 256, 1),       # config 3's first layer
+    (112, 110, 24, 40, 1), (61, 37, 17, 70, 2), (30, 9, 8, 32, 1), (55, 55, 16, 64, 1), (7, 9, 5, 3, 1), (1, 1, 9, 1, 1),
+    (2, 3, 33, 65, 2), (28, 28, 40, 48, 2), (3, 1, 6, 2, 1),
+])
+def test_conv3x3_direct_mfma(lib, dev, oracle, variant, W, H, I, O, s):
+    """The implicit-GEMM 3x3 kernel over the prepared filter bank: oracle (same algorithm, direct order), the
+    float64 closed form, and the filter bank's layout itself.  Signed inputs, so every padding sample matters."""
+    x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
+    n = lib.drhip_conv3x3_direct_filter_floats(I, O)
+    chunks, opad = -(-I // 8), -(-O // 32) * 32
+    assert n == 9 * chunks * 8 * opad
+    F = dev.empty(n)
+    ok(lib, lib.drhip_conv3x3_direct_filter_layout_f32(dev.put(w), F, I, O, None))
+    if variant == 0:
+        expect = np.zeros((9, chunks, opad, 8), np.float32)       # [tap][c/8][o][pos], pos = (c&1)*4 + (c%8)/2
+        for c in range(I):
+            expect[:, c // 8, :O, (c & 1) * 4 + (c % 8) // 2] = w[c].reshape(O, 9).T
+        assert np.array_equal(dev.get(F, expect.shape), expect)
+    want = oracle.conv_direct(x, w, b, (s, s), relu=True)
+    out = dev.empty(want.size)
+    xd, bd = dev.put(x), dev.put(b)
+    ok(lib, lib.drhip_conv3x3_direct_mfma_f32(xd, F, bd, out, W, H, I, O, s, 1, variant, None))
+    got = dev.get(out, want.shape)
+    assert_close(got, want, terms=9 * I)
+    assert_close(got, oracle.conv_f64(x, w, b, stride=(s, s), relu=True), terms=9 * I)
+    want2 = oracle.conv_direct(x, w, None, (s, s), relu=False)      # linear, no bias: sign-sensitive
+    ok(lib, lib.drhip_conv3x3_direct_mfma_f32(xd, F, None, out, W, H, I, O, s, 0, variant, None))
+    assert_close(dev.get(out, want2.shape), want2, terms=9 * I)
+    if variant == 0:
+        assert lib.drhip_conv3x3_direct_mfma_f32(xd, F, None, out, W, H, I, O, 3, 0, 0, None) == -1      # stride 3
+        assert lib.drhip_conv3x3_direct_mfma_f32(xd, F, None, out, W, H, I, O, s, 0, 3, None) == -1      # 3 waves
 
 
 @pytest.mark.parametrize("W,H,I,O,sx,sy", [(224, 224, 3, 64, 2, 2), (33, 31, 3, 9, 2, 2), (17, 13, 1, 5, 1, 1), (20, 18, 4, 70, 1, 2),
