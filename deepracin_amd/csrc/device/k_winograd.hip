@@ -83,13 +83,23 @@ winograd_filter_transform_kernel(const float* __restrict__ w, float* __restrict_
     for (int k = 0; k < 16; ++k) U[wino_u_index(k, c, o, nChunks, Opad)] = u[k];
 }
 
+// Output stores are written through (system-scope store: sc0 sc1) instead of being left dirty in this XCD's L2:
+// the consumer is the next kernel, whose workgroups mostly sit on other XCDs and read from memory anyway, and
+// what is written during the kernel need not be written back when it ends (224x224x64: 23.5 vs 25.0 us).
+__device__ inline void store1_through(float* p, float a) {
+    __hip_atomic_store((unsigned*)p, __float_as_uint(a), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+__device__ inline void store2_through(float* p, float a, float b) {
+    const f32x2 v = {a, b};
+    __hip_atomic_store((unsigned long long*)p, __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // 2x2 store with edge guards; vec2: W even and the base 8-byte aligned.
 __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, int vec2,
                                        float y00, float y01, float y10, float y11) {
     if (vec2) {
-        f32x2 v0 = {y00, y01};
-        *(f32x2*)po = v0;
-        if (oy + 1 < H) { f32x2 v1 = {y10, y11}; *(f32x2*)(po + W) = v1; }
+        store2_through(po, y00, y01);
+        if (oy + 1 < H) store2_through(po + W, y10, y11);
     } else {
         po[0] = y00;
         if (ox + 1 < W) po[1] = y01;
@@ -348,7 +358,7 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
                 if (bias) { const float bv = kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
                 if (relu & kEpiRelu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
                 if (relu & kEpiMaxPool2)        // W, H even: the tile is one window of a 2x2/2 max pool
-                    out[(size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1)] = fmaxf(fmaxf(y00, y01), fmaxf(y10, y11));
+                    store1_through(out + (size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(y00, y01), fmaxf(y10, y11)));
                 else
                     wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, y00, y01, y10, y11);
             }
@@ -534,7 +544,7 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
                 if (bias) { const float bv = biasEarly[q]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
                 if (relu & kEpiRelu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
                 if (relu & kEpiMaxPool2)
-                    out[(size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1)] = fmaxf(fmaxf(y00, y01), fmaxf(y10, y11));
+                    store1_through(out + (size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(y00, y01), fmaxf(y10, y11)));
                 else
                     wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, y00, y01, y10, y11);
             }
@@ -578,7 +588,7 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
     if (relu & kEpiRelu) { s[0] = fmaxf(s[0], 0.f); s[1] = fmaxf(s[1], 0.f); s[2] = fmaxf(s[2], 0.f); s[3] = fmaxf(s[3], 0.f); }
     const int ox = 2 * (tg % tilesX), oy = 2 * (tg / tilesX);
     if (relu & kEpiMaxPool2)
-        out[(size_t)o * ((H >> 1) * (W >> 1)) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1)] = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+        store1_through(out + (size_t)o * ((H >> 1) * (W >> 1)) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
     else
         wino_store_tile(out + (size_t)o * H * W + (size_t)oy * W + ox, W, H, ox, oy, vec2, s[0], s[1], s[2], s[3]);
 }

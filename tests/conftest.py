@@ -42,11 +42,11 @@ def gpu(lib):
     return info
 
 
-def rel_err(a, b):
-    """max |a-b| / max |b|: error relative to the layer's largest magnitude."""
+def rel_err(a, b, floor=1e-30):
+    """max |a-b| / max |b|: error relative to the layer's largest magnitude (at least `floor`)."""
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)
-    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), floor))
 
 
 RTOL, ATOL_OF_MAX = 1e-4, 1e-6
@@ -60,28 +60,30 @@ def atol_factor(terms):
     return max(1.0, (terms / 1024.0) ** 0.5)
 
 
-def elem_err(a, b, terms=0):
-    """Element-wise criterion: worst |a-b| / (1e-4*|b| + 1e-6*atol_factor(terms)*max|b|); <= 1 passes.  Unlike
+def elem_err(a, b, terms=0, floor=1e-30):
+    """Element-wise criterion: worst |a-b| / (1e-4*max(|b|, floor) + 1e-6*atol_factor(terms)*max|b|); <= 1 passes.  Unlike
     rel_err it does not let an element of small magnitude be far off just because the layer has large
     elements elsewhere.  Returns (ratio, flat index of the worst element)."""
     a = np.asarray(a, np.float64).reshape(-1)
     b = np.asarray(b, np.float64).reshape(-1)
     if a.size == 0:
         return 0.0, -1
-    bound = RTOL * np.abs(b) + ATOL_OF_MAX * atol_factor(terms) * max(np.abs(b).max(), 1e-30)
+    bound = RTOL * np.maximum(np.abs(b), floor) + ATOL_OF_MAX * atol_factor(terms) * max(np.abs(b).max(), floor)
     r = np.abs(a - b) / bound
     k = int(np.argmax(r))
     return float(r[k]), k
 
 
-def assert_close(got, want, what="tensor", tol=RTOL, terms=0):
+def assert_close(got, want, what="tensor", tol=RTOL, terms=0, floor=1e-30):
     """Both gates of the per-layer parity bar: max|got-want| / max|want| <= tol (norm-wise) and, element by
     element, |got-want| <= 1e-4*|want| + 1e-6*max|want| (the absolute part widened for sums of more than
-    1024 products, see atol_factor).  The message names the worst element."""
+    1024 products, see atol_factor).  `floor`: a lower limit for max|want| -- the magnitude of the terms
+    that were added up -- for tensors of one or a few elements, whose largest value can itself be the
+    remainder of a cancellation (bias against the convolution sum).  The message names the worst element."""
     got, want = np.asarray(got), np.asarray(want)
     assert got.shape == want.shape, "%s: shape %s vs %s" % (what, got.shape, want.shape)
-    e = rel_err(got, want)
-    r, k = elem_err(got, want, terms)
+    e = rel_err(got, want, floor)
+    r, k = elem_err(got, want, terms, floor)
     msg = "%s: norm-wise %.3g; worst element #%d got %.9g want %.9g (%.3g x its bound)" % (
         what, e, k, got.reshape(-1)[k] if k >= 0 else 0.0, want.reshape(-1)[k] if k >= 0 else 0.0, r)
     assert e <= tol and r <= 1.0, msg

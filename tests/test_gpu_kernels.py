@@ -199,14 +199,15 @@ def test_winograd_conv(lib, dev, oracle, variant, W, H, I, O):
     U, _ = wino_filters(lib, dev, w)
     ws = wino_workspace(lib, dev, W, H, I, O, variant)
     want = oracle.conv_winograd(x, w, b, relu=True)
+    floor = float(np.abs(b).max())                    # tiny tensors: the output can be what is left of bias against conv sum
     out = dev.empty(want.size)
     xd, bd = dev.put(x), dev.put(b)
     for _ in range(2):                       # twice: a split layer must leave its counters at zero
         ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, out, W, H, I, O, 1, variant, ws, None))
         got = dev.get(out, want.shape)
-        assert_close(got, want)
+        assert_close(got, want, floor=floor)
     truth = oracle.conv_f64(x, w, b, relu=True)
-    assert_close(got, truth)
+    assert_close(got, truth, floor=floor)
     # linear, no bias (pre-activation values, sign-sensitive)
     want2 = oracle.conv_winograd(x, w, None, relu=False)
     ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, None, out, W, H, I, O, 0, variant, ws, None))
