@@ -44,6 +44,15 @@ conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, c
     const int o0 = (blockIdx.x / nPT) * 32, p0 = (blockIdx.x % nPT) * 32;
     const int nStages = (I + kC1KC - 1) / kC1KC;
 
+    // The epilogue's bias values are requested now (a load issued there would add a trip to memory to the tail of
+    // the workgroup): with more than one wave, thread tid finishes the elements tid + q*blockDim.x of the tile.
+    float biasEarly[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+        const int idx = tid + q * (int)blockDim.x;
+        biasEarly[q] = (bias && idx < 32 * 32) ? bias[min(o0 + (idx >> 5), O - 1)] : 0.0f;
+    }
+
     f32x16 acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
@@ -99,12 +108,15 @@ conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, c
     for (int r = 0; r < 16; ++r)
         part[(wave * 32 + 8 * (r / 4) + 4 * lhi + (r % 4)) * kC1Pad + l32] = acc[r];
     __syncthreads();
-    for (int idx = tid; idx < 32 * 32; idx += blockDim.x) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {                   // KW >= 2 waves: at most 8 elements per thread
+        const int idx = tid + q * (int)blockDim.x;
+        if (idx >= 32 * 32) break;
         const int ol = idx >> 5, pl = idx & 31;
         const int o = o0 + ol, p = p0 + pl;
         float s = 0.0f;
         for (int k = 0; k < KW; ++k) s += part[(k * 32 + ol) * kC1Pad + pl];
-        if (bias && o < O) s += bias[o];
+        s += biasEarly[q];
         if (relu) s = fmaxf(s, 0.0f);
         if (poolPartials) {
             // sum over the tile's pixels: the 32 lanes of a half wave hold one channel (the trip count
@@ -173,6 +185,17 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
         rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kC1BufferFlags);
     }
 
+    // The epilogue's bias values are requested now: a load issued there would add a trip to memory to the tail of
+    // every workgroup.  Thread tid finishes the elements tid, tid + blockDim.x, ... of the 16x16 tile (at most 4).
+    float biasEarly[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int idx = tid + q * (int)blockDim.x;
+            if (idx < 256) biasEarly[q] = bias[min(o0 + (idx >> 4), O - 1)];
+        }
+    }
+
     f32x4v acc = {0.f, 0.f, 0.f, 0.f};
     float aA[CH], bA[CH][NS], aB[CH], bB[CH][NS];
     // chunk j of this wave = its k-steps wave + KW*(CH*j .. CH*j + CH-1)
@@ -225,13 +248,16 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
 #pragma unroll
     for (int r = 0; r < 4; ++r) part[(wave * 16 + 4 * lk + r) * kC1Pad16 + l16] = acc[r];
     __syncthreads();
-    for (int idx = tid; idx < 16 * 16; idx += blockDim.x) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int idx = tid + q * (int)blockDim.x;
+        if (idx >= 16 * 16) break;
         const int ol = idx >> 4, pl = idx & 15;
         const int o = o0 + ol, p = p0 + pl;
         float s = 0.0f;
         for (int k = 0; k < KW; ++k) s += part[(k * 16 + ol) * kC1Pad16 + pl];
         if (o < O && p < P) {
-            if (bias) s += bias[o];
+            s += biasEarly[q];
             if (relu) s = fmaxf(s, 0.0f);
             out[(size_t)o * P + p] = s;
         }

@@ -466,6 +466,15 @@ conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict
         for (int nt = 0; nt < NT; ++nt) f[nt] = dm_buf_load4(rF, fOff + 4u * (unsigned)(nt * 32 * 8), soff);
     };
 
+    // the epilogue's bias values are requested now: thread tid finishes the elements tid + q*blockDim.x of the tile
+    constexpr int kMaxEpi = 8;                          // (the first 8 of them: all, from two or four waves per workgroup on)
+    float biasEarly[kMaxEpi];
+#pragma unroll
+    for (int q = 0; q < kMaxEpi; ++q) {
+        const int idx = tid + q * (int)blockDim.x;
+        biasEarly[q] = (bias && idx < OB * 32) ? bias[min(o0 + (idx >> 5), O - 1)] : 0.0f;
+    }
+
     f32x16d acc[NT][NA];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
@@ -530,17 +539,24 @@ conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    for (int idx = tid; idx < OB * 32; idx += blockDim.x) {
+    auto finish = [&](int idx, float biasValue) {
         const int ol = idx >> 5, pl = idx & 31;
         const int o = o0 + ol, pp = p0 + pl;
         float v = 0.0f;
         for (int k = 0; k < KW; ++k) v += part[(k * OB + ol) * kDmPartPitch + pl];
         if (o < O && pp < P) {
-            if (bias) v += bias[o];
+            v += biasValue;
             if (relu) v = fmaxf(v, 0.0f);
             out[(size_t)o * P + pp] = v;
         }
+    };
+#pragma unroll
+    for (int q = 0; q < kMaxEpi; ++q) {
+        const int idx = tid + q * (int)blockDim.x;
+        if (idx < OB * 32) finish(idx, biasEarly[q]);
     }
+    for (int idx = tid + kMaxEpi * (int)blockDim.x; idx < OB * 32; idx += blockDim.x)      // one wave per workgroup only
+        finish(idx, bias ? bias[min(o0 + (idx >> 5), O - 1)] : 0.0f);
 }
 
 template <int OCT>
