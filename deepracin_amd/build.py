@@ -22,7 +22,10 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-fPIC", "-std=c++17", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(CSRC, "device"),
           "-I" + os.path.join(CSRC, "host"), "-Wall", "-Wno-unused-function"]
 # Packed-fp32 VALU forms are kept out of the generated code on purpose.
-DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# The first 16 dwords of every kernel's arguments arrive in SGPRs with the wave instead of through a scalar load at
+# its start (gfx950 kernarg preload): about 0.1 us off each of the 19-23 launches of a batch-1 pass.
+DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 
 
 def sources():
