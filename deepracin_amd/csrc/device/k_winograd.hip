@@ -379,14 +379,18 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
 // A workgroup owns 16 tiles x OB = 16*NB output channels.
 typedef float f32x4acc __attribute__((ext_vector_type(4)));
 
-template <int NB>
-__global__ void __launch_bounds__(kWinoThreads)
+// KW wave sets of four waves (KW = 1, 2) take the stages round-robin and meet in LDS in the epilogue, set 0 first:
+// a stage is only 8*NB short MFMAs long, less than a load takes to arrive, so a single wave per SIMD waits for its
+// operands in every stage; with two waves per SIMD the prefetch of a wave has two stages of matrix work to land
+// (14x14, 64 -> 256: 5.1 vs 5.4 us; four sets were measured slower again).
+template <int NB, int KW>
+__global__ void __launch_bounds__(kWinoThreads * KW)
 winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ U,
                            const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
                            int W, int H, int I, int O, int tilesX, int T, int nTB, int nBlocks,
                            int chunksPerSplit, int relu, int vec2) {
     constexpr int TB = 16, OB = 16 * NB, KC = kWinoKC;
-    extern __shared__ float P[];                    // epilogue only: [4 rows][2][OB o][16 t] floats
+    extern __shared__ float P[];                    // epilogue only: [KW sets][4 rows][2][OB o][16 t] floats
 
     const int perXcd = gridDim.x / kXcds;
     const int logical = (blockIdx.x % kXcds) * perXcd + blockIdx.x / kXcds;
@@ -396,7 +400,9 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
     const int split = blockIdx.y, nSplits = gridDim.y;
 
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // = row of the transform
+    const int waveId = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = waveId & 3;                    // = row of the transform
+    const int kset = waveId >> 2;                   // which of the KW wave sets
     const int l16 = lane & 15, lk = lane >> 4;
     const int plane = H * W;
     const int nChunksAll = (I + KC - 1) / KC;
@@ -440,10 +446,12 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
         for (int nb = 0; nb < NB; ++nb) f[nb] = buf_load4(rU, fOff + 4u * (unsigned)(nb * 16 * 8), soff);
     };
 
-    float biasEarly[OB / 16];
+    constexpr int EO = 16 * KW;                     // output channels finished per pass of the epilogue
+    constexpr int NQ = (OB + EO - 1) / EO;
+    float biasEarly[NQ];
     if (bias && gridDim.y == 1) {
 #pragma unroll
-        for (int q = 0; q < OB / 16; ++q) biasEarly[q] = bias[min(o0 + (tid >> 4) + 16 * q, O - 1)];
+        for (int q = 0; q < NQ; ++q) biasEarly[q] = bias[min(o0 + (tid >> 4) + EO * q, O - 1)];
     }
 
     f32x4acc acc[4][NB];
@@ -455,12 +463,12 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
     float raw[2][8];
     f32x4 f[4][NB];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) load_rows_ranged(raw[ks], chBegin * KC + 4 * ks);
+    for (int ks = 0; ks < 2; ++ks) load_rows_ranged(raw[ks], (chBegin + kset) * KC + 4 * ks);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) load_filters(f[e], e, chBegin);
+    for (int e = 0; e < 4; ++e) load_filters(f[e], e, min(chBegin + kset, nChunksAll - 1));
 
     auto stage = [&](int ch, auto plainNext) {
-        const int next = min(ch + 1, nChunksAll - 1);
+        const int next = min(ch + KW, nChunksAll - 1);
         float b[2][4];                              // [k-step][xi within the row]
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
@@ -490,8 +498,8 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
                         acc[e][nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, b[ks][e], acc[e][nb], 0, 0, 0);
                     }
                 if (eg == 0) {
-                    if constexpr (decltype(plainNext)::value) load_rows_plain(raw[ks], (ch + 1) * KC + 4 * ks);
-                    else load_rows_ranged(raw[ks], (ch + 1) * KC + 4 * ks);
+                    if constexpr (decltype(plainNext)::value) load_rows_plain(raw[ks], (ch + KW) * KC + 4 * ks);
+                    else load_rows_ranged(raw[ks], (ch + KW) * KC + 4 * ks);
                 } else {
                     load_filters(f[ks], ks, next);
                 }
@@ -502,10 +510,10 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
         load_filters(f[3], 3, next);
         __builtin_amdgcn_sched_barrier(0);
     };
-    const int chMain = max(chBegin, min(chEnd, I / KC - 1));
-    int ch = chBegin;
-    for (; ch < chMain; ++ch) stage(ch, std::true_type{});
-    for (; ch < chEnd; ++ch) stage(ch, std::false_type{});
+    const int chMain = min(chEnd, I / KC - KW);
+    int ch = chBegin + kset;
+    for (; ch < chMain; ch += KW) stage(ch, std::true_type{});
+    for (; ch < chEnd; ch += KW) stage(ch, std::false_type{});
 
     // ---- epilogue: right factor in registers, rows meet in LDS, left factor, bias, ReLU, store ----
 #pragma unroll
@@ -514,8 +522,8 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
         for (int r = 0; r < 4; ++r) {
             const float m0 = acc[0][nb][r], m1 = acc[1][nb][r], m2 = acc[2][nb][r], m3 = acc[3][nb][r];
             const int ol = 16 * nb + 4 * lk + r;
-            P[((wave * 2 + 0) * OB + ol) * TB + l16] = m0 + m1 + m2;
-            P[((wave * 2 + 1) * OB + ol) * TB + l16] = m1 - m2 + m3;
+            P[(((kset * 4 + wave) * 2 + 0) * OB + ol) * TB + l16] = m0 + m1 + m2;
+            P[(((kset * 4 + wave) * 2 + 1) * OB + ol) * TB + l16] = m1 - m2 + m3;
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
@@ -529,13 +537,19 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
     const int ox = eTileOk ? 2 * (etg % tilesX) : 0, oy = eTileOk ? 2 * (etg / tilesX) : 0;
     f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
 #pragma unroll
-    for (int q = 0; q < OB / 16; ++q) {
-        const int ol = eo + 16 * q, o = o0 + ol;
+    for (int q = 0; q < NQ; ++q) {
+        const int ol = eo + EO * q, o = o0 + ol;
+        if (ol >= OB) break;                        // (EO can exceed OB: 16 channels, four wave sets)
         float p[4][2];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             p[r][0] = P[((r * 2 + 0) * OB + ol) * TB + et];
             p[r][1] = P[((r * 2 + 1) * OB + ol) * TB + et];
+#pragma unroll
+            for (int ksx = 1; ksx < KW; ++ksx) {    // the other wave sets' shares of the channel sum, in set order
+                p[r][0] += P[(((ksx * 4 + r) * 2 + 0) * OB + ol) * TB + et];
+                p[r][1] += P[(((ksx * 4 + r) * 2 + 1) * OB + ol) * TB + et];
+            }
         }
         float y00 = p[0][0] + p[1][0] + p[2][0], y01 = p[0][1] + p[1][1] + p[2][1];
         float y10 = p[1][0] - p[2][0] + p[3][0], y11 = p[1][1] - p[2][1] + p[3][1];
@@ -596,12 +610,14 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
 // variant = output channels per workgroup (low 4 bits: 1 -> 32, 2 -> 64, 3 -> 128)
 //         | log2(number of input-channel splits) << 4
 //         | 0x100: 16-tile blocks (then the low 4 bits mean 1 -> 16, 2 -> 32, 3 -> 64 channels)
-//         | 0x400: eight waves per workgroup, two wave sets sharing the stages (32-tile blocks of 32 or 64 channels)
+//         | 0x400: eight waves per workgroup, two wave sets sharing the stages (32-tile blocks of 32 or 64 channels,
+//                  or 16-tile blocks)
 struct WinoCfg { int nt, splits, tb, waveSets; };
 
 static bool wino_variant(int variant, WinoCfg* c) {
     c->waveSets = (variant & 0x400) ? 2 : 1;
-    if (c->waveSets == 2 && ((variant & 0x300) || (variant & 0xf) > 2)) return false;
+    if (variant >> 11) return false;
+    if (c->waveSets == 2 && !(variant & 0x100) && (variant & 0xf) > 2) return false;
     variant &= ~0x400;
     const int lg = (variant >> 4) & 0xf;
     if (lg > 6 || (variant >> 9)) return false;
@@ -658,8 +674,11 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
         if (c.waveSets != 2 || NT > 2)
             launch((winograd_f23_mfma_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
                    in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
-    } else
-        launch((winograd_f23_mfma16_kernel<NT>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
+    } else if (c.waveSets == 2)
+        launch((winograd_f23_mfma16_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
+               in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
+    else
+        launch((winograd_f23_mfma16_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
                in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
     if (g.splits > 1) {
@@ -688,7 +707,8 @@ extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     // Small layers (SqueezeNet's expand convolutions: <= 8 stages, a few dozen 32x32 panels) are bound
     // by the latency of one workgroup, not by throughput: 16x16 blocks, unsplit, one launch
     // (in a replayed launch graph 4.2-5.8 us per layer against 5.1-7.1 us for the 32x32 forms).
-    if (ceil_div(T, 32) * ceil_div(O, 32) < cus / 2 && ceil_div(I, kWinoKC) <= 16) return 0x101;
+    if (ceil_div(T, 32) * ceil_div(O, 32) < cus / 2 && ceil_div(I, kWinoKC) <= 16)
+        return (ceil_div(I, kWinoKC) >= 6 && T <= 64) ? 0x501 : 0x101;      // 14x14 maps with 6+ stages: two wave sets
     const int code = (O > 32 && T >= 8192) ? 2 : 1;
     const int panels = ceil_div(T, 32) * ceil_div(O, code == 2 ? 64 : 32);
     const int nChunks = ceil_div(I, kWinoKC);

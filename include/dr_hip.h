@@ -155,7 +155,7 @@ int drhip_winograd_filter_transform_f32(const float* w /* [I][O][3][3] */, float
  * `variant` is the configuration chosen by the scheduler: low 4 bits = output channels per
  * workgroup (1: 32, 2: 64, 3: 128), bits 4-7 = log2 of the number of input-channel splits, 0x100 =
  * blocks of 16 tiles (channels per workgroup then 16, 32, 64), 0x400 = eight waves per workgroup (two
- * wave sets that take alternate 8-channel stages; 32-tile blocks of 32 or 64 channels only); 0 lets
+ * wave sets that take alternate 8-channel stages; not with 32-tile blocks of 128 channels); 0 lets
  * the launcher pick.  The input must be smaller than 2 GiB (32-bit byte offsets).  A variant that splits the
  * input channels needs `workspace` of drhip_conv3x3_winograd_workspace_floats(...) floats (scratch,
  * no initialisation needed; two launches: partial tiles, then their sum in split order); otherwise

@@ -187,7 +187,7 @@ def test_winograd_filter_transform(lib, dev, oracle):
 
 
 @pytest.mark.parametrize("variant", [1, 2, 3, 0x11, 0x21, 0x12, 0x33, 0x101, 0x102, 0x103, 0x111, 0x122,
-                                     0x401, 0x402, 0x411, 0x432])
+                                     0x401, 0x402, 0x411, 0x432, 0x501, 0x502, 0x503, 0x512])
 @pytest.mark.parametrize("W,H,I,O", [
     (56, 56, 64, 64),        # config 1
     (55, 55, 16, 64),        # fire expand3x3: odd size, two stages of 8 channels
@@ -214,7 +214,7 @@ def test_winograd_conv(lib, dev, oracle, variant, W, H, I, O):
     assert_close(dev.get(out, want2.shape), want2)
 
 
-@pytest.mark.parametrize("variant", [1, 2, 0x11, 0x22, 0x101, 0x112, 0x401, 0x412])
+@pytest.mark.parametrize("variant", [1, 2, 0x11, 0x22, 0x101, 0x112, 0x401, 0x412, 0x502])
 @pytest.mark.parametrize("W,H,I,O", [(56, 56, 64, 64), (28, 12, 24, 40), (2, 2, 1, 1), (224, 224, 3, 64)])
 def test_winograd_fused_maxpool(lib, dev, oracle, variant, W, H, I, O):
     """Epilogue flag 2: the kernel stores the 2x2/2 maximum of every output tile -- bit for bit what
