@@ -54,7 +54,7 @@ static FcPlan fc_plan(int K, int N) {
     p.panels = ceil_div(N, p.cbw);
     const int target = 4 * num_cu();                 // workgroups wanted in flight
     int slices = ceil_div(target, p.panels);
-    const int maxSlices = ceil_div(K, 2 * kWave);    // at least two 64-row chunks per workgroup
+    const int maxSlices = ceil_div(K, 4 * kWave);    // at least 256 rows per workgroup (4096 x 4096: 13.7 us with 16 slices, 14.8 with 32)
     if (slices > maxSlices) slices = maxSlices;
     if (slices < 1) slices = 1;
     p.rowsPerSlice = ceil_div(ceil_div(K, slices), kWave) * kWave;   // whole chunks

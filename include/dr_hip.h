@@ -254,7 +254,7 @@ int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, const float*
  * looked up by drhip_init, which must have run for the current device).  The call allocates and
  * frees nothing.  Shapes whose partial sums exceed drhip_fc_noalloc_max_scratch_floats() floats
  * (drhip_fc_scratch_floats(K,N) tells) are refused with DRHIP_EINVAL; VGG16's three layers need
- * 229376, 131072 and 32000.  All calls on one GPU share the array: calls that may overlap (different
+ * 229376, 65536 and 16000.  All calls on one GPU share the array: calls that may overlap (different
  * streams, or graph branches) race on it; calls on one stream are safe.  Refused while
  * drhip_timing_begin is active. */
 size_t drhip_fc_noalloc_max_scratch_floats(void);
