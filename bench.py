@@ -21,7 +21,9 @@ of 20 passes is a few milliseconds long and a single sample of it says little), 
                  profiles/) and `mfma_busy_frac` = issued_tflops / 157.3, the share of the data-sheet
                  matrix peak the pipe was issuing at; the >= 50 % target is judged on `mfma_busy_frac`.
                  `mfma_busy_frac_counters` is the same share from SQ_VALU_MFMA_BUSY_CYCLES of the
-                 committed rocprofv3 run (profiles/counters.json), null when there is none.  Device
+                 committed rocprofv3 run (profiles/counters.json: busy cycles per SIMD / (this run's device
+                 time x 2.4 GHz)), `mfma_busy_frac_profiled` the share over the profiler's own, longer,
+                 kernel durations; null when there is no such run.  Device
                  times come from HIP events on the graph's own stream in a separate instrumented region:
                  with profilingGPU set the library attaches a start and a stop event to every kernel
                  launch, so a launch's span is the kernel alone, as in a rocprofv3 kernel trace.
@@ -152,7 +154,7 @@ def measure(workload, seed, steps, warmup, blocks=BLOCKS, instrument=True, env_v
 
         # wall-clock rate of the loop the reference's users run: feed (H2D over PCIe), pass, download of the output
         feed_idx, feed_arr = next(iter(feeds.items()))
-        n_e2e = max(steps, 20)
+        n_e2e = max(steps, 100)
         for _ in range(3):
             configs.feed_chw(nodes[feed_idx], feed_arr); lib.dR_apply(g.ptr); configs.fetch_chw(g)
         t0 = time.perf_counter()
@@ -247,8 +249,12 @@ def analyse(lib, m, workload, counters):
                     "flops_per_launch": gk["flops"] / max(gk["launches"], 1)}
         if dominant == "winograd":
             issued = gk["issued"] / (gk["ms"] * 1e-3) / 1e12
+            # counters of the committed rocprofv3 run: busy cycles per SIMD over THIS run's device time (the profiler's own
+            # timestamps run ~10 % long), and the share under the profiler itself
+            cyc = rec.get("mfma_busy_cycles_per_simd")
             roofline.update({"issued_tflops": round(issued, 3), "mfma_busy_frac": round(issued / PEAK_MFMA_F32_TFLOPS, 4),
-                             "mfma_busy_frac_counters": rec.get("mfma_busy_frac"),
+                             "mfma_busy_frac_counters": round(cyc / (gk["ms"] * 1e3 * PEAK_CLOCK_GHZ * 1e3), 4) if cyc else None,
+                             "mfma_busy_frac_profiled": rec.get("mfma_busy_frac"),
                              "target": "mfma_busy_frac >= 0.50"})
         if rec.get("measured"):
             roofline["counters_measured"] = rec["measured"]
