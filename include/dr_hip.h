@@ -88,12 +88,16 @@ int drhip_fill_f32(float* dst, float value, size_t n, void* stream);
 /* Staged transfers for the per-image copies of a serving loop (the feed of dR_feedData, the logits of
  * dR_downloadArray).  A staging object owns pinned host memory (hipHostMalloc): an upload area of
  * `upload_bytes` and a 64 KiB download area.  drhip_upload_staged copies the caller's (pageable) array
- * into the upload area and starts one transfer from there; it returns when the caller's array has been
+ * into the upload area and starts one transfer from there (up to 4 MiB: a kernel that reads the pinned
+ * area, which starts sooner than the DMA engine; DR_UPLOAD_KERNEL=0 in the environment or larger arrays:
+ * hipMemcpyAsync); it returns when the caller's array has been
  * read (the array may be reused), NOT when the data is on the device: the transfer is ordered on
  * `stream` before whatever is enqueued next, and a following staged upload waits for it.
  * drhip_download_staged blocks like drhip_download; the data comes through the download area, stored
- * there by a small copy kernel (the area is mapped into the device's address space).  One staging
- * object serves one stream at a time.  Replace the blocking clEnqueueWriteBuffer / clEnqueueReadBuffer
+ * there by a small copy kernel (the area is mapped into the device's address space) that raises a flag
+ * behind the data; the host watches the flag for up to DR_SPIN_US microseconds (default 1000; 0 = never)
+ * before it waits for the stream the ordinary way - the flag is seen some 10 us before the stream's own
+ * completion reaches the host.  One staging object serves one stream at a time.  Replace the blocking clEnqueueWriteBuffer / clEnqueueReadBuffer
  * of dR_uploadArray / dR_downloadArray (src/dR_clwrap.c:1079-1190) on the per-image path. */
 int    drhip_staging_create(void** handle, size_t upload_bytes);
 int    drhip_staging_destroy(void* handle);

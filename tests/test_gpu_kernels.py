@@ -456,6 +456,46 @@ def test_softmax(lib, dev, oracle):
     assert_close(dev.get(y, (3,)), oracle.softmax_f64(big))
 
 
+@pytest.mark.parametrize("env", [{}, {"DR_SPIN_US": "0"}, {"DR_UPLOAD_KERNEL": "0"}])
+def test_staged_transfers_carry_every_byte(lib, dev, env):
+    """Uploads through the pinned area (by kernel and by the DMA engine: odd destination offsets and sizes
+    take the latter) and downloads through the flagged copy kernel, many times over with new contents and
+    sizes each time: a flag seen before its data, or data left in the area from the call before, would show."""
+    import os
+    os.environ.update(env)
+    try:
+        h = ctypes.c_void_p()
+        ok(lib, lib.drhip_staging_create(ctypes.byref(h), 1 << 20))
+    finally:
+        for k in env:
+            os.environ.pop(k, None)
+    assert lib.drhip_staging_upload_capacity(h) == 1 << 20 and lib.drhip_staging_download_capacity(h) == 65536
+    rng = np.random.default_rng(11)
+    buf = dev.empty(1 << 18)
+    vp = ctypes.c_void_p
+    try:
+        for it in range(300):
+            n = int(rng.choice([1, 3, 4, 250, 1000, 4096, 16383, 16384]))
+            off = int(rng.integers(0, 64)) * int(rng.choice([1, 4]))          # floats; some 16-byte aligned, some not
+            a = rng.standard_normal(n).astype(np.float32) + it
+            ok(lib, lib.drhip_upload_staged(h, buf, 4 * off, a.ctypes.data_as(vp), a.nbytes, None))
+            a_copy = a.copy()
+            a[...] = np.nan                                                    # the caller's array is free again
+            back = np.full(n, -1.0, np.float32)
+            ok(lib, lib.drhip_download_staged(h, back.ctypes.data_as(vp), buf, 4 * off, back.nbytes, None))
+            assert np.array_equal(back, a_copy), (it, n, off)
+        # bytes that are not whole floats go through the DMA engine both ways
+        raw = rng.integers(0, 256, 1001, dtype=np.uint8)
+        ok(lib, lib.drhip_upload_staged(h, buf, 3, raw.ctypes.data_as(vp), raw.nbytes, None))
+        got = np.zeros_like(raw)
+        ok(lib, lib.drhip_download_staged(h, got.ctypes.data_as(vp), buf, 3, got.nbytes, None))
+        assert np.array_equal(got, raw)
+        assert lib.drhip_download_staged(h, got.ctypes.data_as(vp), buf, 0, 65537, None) == -1
+        assert lib.drhip_upload_staged(h, buf, 0, raw.ctypes.data_as(vp), (1 << 20) + 1, None) == -1
+    finally:
+        lib.drhip_staging_destroy(h)
+
+
 def test_copy3d_and_scalar(lib, dev, oracle):
     x = rnd(6, 9, 11)
     out = dev.empty(3 * 4 * 5)
