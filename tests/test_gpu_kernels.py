@@ -5,6 +5,7 @@ Tolerances (north star): fp32 layers max relative error <= 1e-4, measured as
 max|gpu - oracle| / max|oracle| over the layer; pooling values and max-indices bit-exact.
 """
 import ctypes
+import os
 
 import numpy as np
 import pytest
@@ -513,13 +514,15 @@ def test_copy3d_and_scalar(lib, dev, oracle):
 # width the kernels use, single rows / columns / channels included.
 
 def _sweep(seed, count, draw):
+    """`count` seeded draws; DR_SWEEP_SCALE=n in the environment multiplies the count for a one-off wider run."""
     rng = np.random.default_rng(seed)
-    return [draw(rng) for _ in range(count)]
+    return [draw(rng) for _ in range(count * int(os.environ.get("DR_SWEEP_SCALE", "1")))]
 
 
-@pytest.mark.parametrize("W,H,I,O,variant", _sweep(11, 24, lambda r: (
+@pytest.mark.parametrize("W,H,I,O,variant", _sweep(11, 40, lambda r: (
     int(r.integers(1, 41)), int(r.integers(1, 41)), int(r.integers(1, 41)), int(r.integers(1, 71)),
-    int(r.choice([0, 1, 2, 3, 0x11, 0x12, 0x21, 0x31, 0x101, 0x102, 0x103, 0x111, 0x121]))))
+    int(r.choice([0, 1, 2, 3, 0x11, 0x12, 0x21, 0x31, 0x101, 0x102, 0x103, 0x111, 0x121,
+                  0x401, 0x402, 0x411, 0x422, 0x501, 0x502, 0x503, 0x511, 0x521]))))
     + [(1, 37, 9, 31, 0x11), (37, 1, 8, 32, 1), (3, 3, 64, 33, 0x21), (40, 2, 17, 1, 2)])
 def test_winograd_sweep(lib, dev, oracle, W, H, I, O, variant):
     x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
@@ -547,6 +550,37 @@ def test_conv_direct_sweep(lib, dev, oracle, W, H, I, O, kw, kh, sx, sy):
     got = dev.get(out, want.shape)
     assert_close(got, want)
     assert_close(got, oracle.conv_f64(x, w, b, stride=(sx, sy)))
+
+
+@pytest.mark.parametrize("W,H,I,O,s,variant", _sweep(16, 32, lambda r: (
+    int(r.integers(1, 41)), int(r.integers(1, 41)), int(r.integers(1, 41)), int(r.integers(1, 71)), int(r.integers(1, 3)),
+    int(r.choice([0, 1, 2, 4, 8, 0x11, 0x12, 0x14, 0x18]))))
+    + [(1, 40, 9, 31, 1, 0x12), (40, 1, 8, 33, 2, 4), (3, 3, 64, 65, 1, 8), (2, 2, 7, 1, 2, 0x11)])
+def test_conv3x3_direct_mfma_sweep(lib, dev, oracle, W, H, I, O, s, variant):
+    if W // s == 0 or H // s == 0:
+        pytest.skip("empty output")
+    x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
+    F = dev.empty(lib.drhip_conv3x3_direct_filter_floats(I, O))
+    ok(lib, lib.drhip_conv3x3_direct_filter_layout_f32(dev.put(w), F, I, O, None))
+    relu = (W + H + I + O) & 1
+    want = oracle.conv_direct(x, w, b, (s, s), relu=bool(relu))
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_conv3x3_direct_mfma_f32(dev.put(x), F, dev.put(b), out, W, H, I, O, s, relu, variant, None))
+    got = dev.get(out, want.shape)
+    assert_close(got, want, terms=9 * I)
+    assert_close(got, oracle.conv_f64(x, w, b, stride=(s, s), relu=bool(relu)), terms=9 * I)
+
+
+@pytest.mark.parametrize("Win,Hin,I,O", _sweep(17, 20, lambda r: (
+    int(r.integers(1, 60)), int(r.integers(1, 60)), int(r.integers(1, 140)), int(r.integers(1, 70)))))
+def test_conv1x1_with_pooled_input_sweep(lib, dev, oracle, Win, Hin, I, O):
+    x, w, b = rnd(I, Hin, Win), rnd(I, O, 1, 1, scale=np.sqrt(2.0 / I)), rnd(O, scale=0.01)
+    pooled = oracle.pool(x, (3, 3, 1), (2, 2, 1), 0)
+    relu = (Win + Hin + I + O) & 1
+    want = oracle.conv1x1(pooled, w, b, relu=bool(relu))
+    out = dev.empty(want.size)
+    ok(lib, lib.drhip_conv1x1_pooled3s2_f32(dev.put(x), dev.put(w), dev.put(b), out, Win, Hin, I, O, relu, None))
+    assert_close(dev.get(out, want.shape), want, terms=I)
 
 
 @pytest.mark.parametrize("P,I,O,variant", _sweep(13, 20, lambda r: (
