@@ -564,10 +564,12 @@ def _random_spec(seed):
     return spec, x, some
 
 
-@pytest.mark.parametrize("seed", range(48))
+@pytest.mark.parametrize("seed", range(48 * int(os.environ.get("DR_SWEEP_SCALE", "1"))))    # (a one-off wider run: DR_SWEEP_SCALE=n)
 def test_random_topologies(oracle, gpu, seed):
     spec, x, some = _random_spec(1000 + seed)
     want = oracle.run_spec(spec, {0: x})
+    if not all(np.isfinite(a).all() for a in want if a is not None):
+        pytest.skip("degenerate draw: a Normalization node met a constant tensor (deviation 0)")
     for outs in (some, [i for i in range(1, len(spec))]):
         with dr.Environment() as env:
             g = env.create_graph()
