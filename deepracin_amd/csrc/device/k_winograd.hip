@@ -660,11 +660,14 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
         if constexpr (NT <= 2) {
             if (c.waveSets == 2) {
                 // more than 64 KiB of dynamic LDS has to be asked for once per kernel
-                static bool raised = false;
-                if (2 * ldsBytes > 65536 && !raised) {
+                // (the attribute belongs to the kernel's code object on ONE device)
+                static bool raised[64] = {};
+                int device = 0;
+                if (int rc = check(hipGetDevice(&device), "hipGetDevice")) return rc;
+                if (2 * ldsBytes > 65536 && !(device >= 0 && device < 64 && raised[device])) {
                     if (int rc = check(hipFuncSetAttribute((const void*)winograd_f23_mfma_kernel<NT, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * ldsBytes)),
                                        "hipFuncSetAttribute(max dynamic LDS)")) return rc;
-                    raised = true;
+                    if (device >= 0 && device < 64) raised[device] = true;
                 }
             }
             if (c.waveSets == 2)
