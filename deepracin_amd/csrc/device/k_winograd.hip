@@ -711,7 +711,8 @@ extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     // by the latency of one workgroup, not by throughput: 16x16 blocks, unsplit, one launch
     // (in a replayed launch graph 4.2-5.8 us per layer against 5.1-7.1 us for the 32x32 forms).
     if (ceil_div(T, 32) * ceil_div(O, 32) < cus / 2 && ceil_div(I, kWinoKC) <= 16)
-        return (ceil_div(I, kWinoKC) >= 6 && T <= 64) ? 0x501 : 0x101;      // 14x14 maps with 6+ stages: two wave sets
+        // 6+ stages and at most one workgroup per CU (14x14 maps; 56x56 64->64: 5.3 vs 5.5 us): two wave sets
+        return (ceil_div(I, kWinoKC) >= 6 && ceil_div(T, 16) * ceil_div(O, 16) <= cus) ? 0x501 : 0x101;
     const int code = (O > 32 && T >= 8192) ? 2 : 1;
     const int panels = ceil_div(T, 32) * ceil_div(O, code == 2 ? 64 : 32);
     const int nChunks = ceil_div(I, kWinoKC);
