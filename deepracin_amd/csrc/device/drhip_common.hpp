@@ -65,6 +65,19 @@ inline void launch(Kernel kernel, dim3 grid, dim3 block, size_t ldsBytes, hipStr
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// Division by a number known at launch time, as a multiplication (Granlund & Montgomery): with
+// l = ceil(log2 d) and mul = floor(2^32 (2^l - d) / d) + 1, n / d = (mulhi(n, mul) + n) >> l for every n < 2^31.
+// A hardware integer division is some 30 dependent instructions, and in the short kernels of a batch-1 pass
+// those in front of a workgroup's first loads are part of every layer's latency (~0.1 us per kernel).
+struct FastDiv { unsigned d, mul, shift; };
+inline FastDiv make_fastdiv(int d) {                 // d >= 1
+    unsigned l = 0;
+    while ((1ull << l) < (unsigned long long)d) ++l;
+    const unsigned long long m = ((1ull << 32) * ((1ull << l) - (unsigned long long)d)) / (unsigned long long)d + 1;
+    return FastDiv{(unsigned)d, (unsigned)m, l};
+}
+__device__ inline int fast_div(int n, const FastDiv& f) { return (int)((__umulhi((unsigned)n, f.mul) + (unsigned)n) >> f.shift); }
+
 // Element `row` of an activation vector that a split GEMV left as partial sums: slices added in
 // order, then bias and ReLU -- bit for bit what the GEMV's finishing kernel stores.
 __device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {

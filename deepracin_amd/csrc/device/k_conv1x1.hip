@@ -41,7 +41,7 @@ conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, c
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int KW = blockDim.x >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
-    const int o0 = (blockIdx.x / nPT) * 32, p0 = (blockIdx.x % nPT) * 32;
+    const int o0 = blockIdx.y * 32, p0 = blockIdx.x * 32;      // (a 2-D grid: an integer division here delays the first loads)
     const int nStages = (I + kC1KC - 1) / kC1KC;
 
     // The epilogue's bias values are requested now (a load issued there would add a trip to memory to the tail of
@@ -155,7 +155,7 @@ constexpr unsigned kC1BufferFlags = 0x00020000u;    // dword 3 of a gfx9 raw buf
 template <bool POOL>
 __global__ void __launch_bounds__(POOL ? 512 : 1024)
 conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
-                      float* __restrict__ out, int P, int I, int O, int nPT, int relu, int Win, int Hin, int Wp) {
+                      float* __restrict__ out, int P, int I, int O, int nPT, int relu, int Win, int Hin, FastDiv Wpd) {
     extern __shared__ float part[];                 // [KW][16][kC1Pad16]
     constexpr int CH = POOL ? 4 : kC1Chunk;         // k-steps per chunk
     constexpr int NS = POOL ? 12 : 1;               // floats loaded per B operand (3 window rows of 4)
@@ -163,7 +163,7 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int KW = blockDim.x >> 6;
     const int l16 = lane & 15, lk = lane >> 4;
-    const int o0 = (blockIdx.x / nPT) * 16, p0 = (blockIdx.x % nPT) * 16;
+    const int o0 = blockIdx.y * 16, p0 = blockIdx.x * 16;    // (a 2-D grid: an integer division here delays the first loads)
     const int nK = (I + 3) / 4;                     // k-steps of 4 channels
     const int oL = min(o0 + l16, O - 1), pL = min(p0 + l16, P - 1);
     const bool oOk = o0 + l16 < O, pOk = p0 + l16 < P;
@@ -175,7 +175,7 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
     bool colIn[3] = {true, true, true}, rowIn[3] = {true, true, true};
     __amdgpu_buffer_rsrc_t rIn;
     if constexpr (POOL) {
-        const int py = pL / Wp, px = pL - py * Wp;
+        const int py = fast_div(pL, Wpd), px = pL - py * (int)Wpd.d;
 #pragma unroll
         for (int d = 0; d < 3; ++d) {
             rowIn[d] = 2 * py + d < Hin;
@@ -231,7 +231,7 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
             acc = __builtin_amdgcn_mfma_f32_16x16x4f32((cOk && oOk) ? a[u] : 0.0f, (cOk && pOk) ? bv : 0.0f, acc, 0, 0, 0);
         }
     };
-    const int mine = (nK - wave + KW - 1) / KW;                 // k-steps of this wave (>= 0)
+    const int mine = (nK - wave + KW - 1) >> (31 - __builtin_clz(KW));     // k-steps of this wave (>= 0); KW is a power of two
     const int chunks = (mine + CH - 1) / CH;
     // Two buffers, the next chunk always on its way.  The loop leaves right after the last real
     // chunk: the loads issued beyond it (clamped addresses) are never waited for.
@@ -299,14 +299,16 @@ extern "C" int drhip_conv1x1_f32(const float* in, const float* w, const float* b
         DRHIP_REQUIRE((variant >> 9) == 0, "drhip_conv1x1_f32: unknown variant %#x", variant);
         DRHIP_REQUIRE(kw == 1 || kw == 2 || kw == 4 || kw == 8 || kw == 16, "drhip_conv1x1_f32: unknown variant %#x (16x16 tiles: 1..16 waves)", variant);
         const int nPT16 = ceil_div(P, 16), nOT16 = ceil_div(O, 16);
-        launch(conv1x1_mfma16_kernel<false>, dim3(nPT16 * nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
-               in, w, bias, out, P, I, O, nPT16, relu, 0, 0, 0);
+        DRHIP_REQUIRE(nOT16 <= 65535, "drhip_conv1x1_f32: too many output channels for 16x16 tiles (%d)", O);
+        launch(conv1x1_mfma16_kernel<false>, dim3(nPT16, nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
+               in, w, bias, out, P, I, O, nPT16, relu, 0, 0, make_fastdiv(1));
         return launched("conv1x1_mfma16_kernel");
     }
     DRHIP_REQUIRE(variant == 1 || variant == 2 || variant == 4 || variant == 8, "drhip_conv1x1_f32: unknown variant %d (waves per tile: 1, 2, 4, 8)", variant);
     const int nPT = ceil_div(P, 32), nOT = ceil_div(O, 32);
+    DRHIP_REQUIRE(nOT <= 65535, "drhip_conv1x1_f32: too many output channels (%d)", O);
     const size_t ldsBytes = variant > 1 ? (size_t)variant * 32 * kC1Pad * sizeof(float) : 0;
-    launch(conv1x1_mfma_kernel, dim3(nPT * nOT), dim3(64 * variant), ldsBytes, as_stream(stream),
+    launch(conv1x1_mfma_kernel, dim3(nPT, nOT), dim3(64 * variant), ldsBytes, as_stream(stream),
                        in, w, bias, out, (float*)nullptr, P, I, O, nPT, relu);
     return launched("conv1x1_mfma_kernel");
 }
@@ -324,7 +326,8 @@ extern "C" int drhip_conv1x1_poolsum_f32(const float* in, const float* w, const 
     int kw = 2;
     while (kw < 8 && stages >= 4 * kw && tiles * kw < 8 * num_cu()) kw *= 2;
     const int nPT = ceil_div(P, 32), nOT = ceil_div(O, 32);
-    launch(conv1x1_mfma_kernel, dim3(nPT * nOT), dim3(64 * kw), (size_t)kw * 32 * kC1Pad * sizeof(float), as_stream(stream),
+    DRHIP_REQUIRE(nOT <= 65535, "drhip_conv1x1_poolsum_f32: too many output channels (%d)", O);
+    launch(conv1x1_mfma_kernel, dim3(nPT, nOT), dim3(64 * kw), (size_t)kw * 32 * kC1Pad * sizeof(float), as_stream(stream),
            in, w, bias, (float*)nullptr, partials, P, I, O, nPT, relu);
     return launched("conv1x1_mfma_kernel");
 }
@@ -341,7 +344,8 @@ extern "C" int drhip_conv1x1_pooled3s2_f32(const float* in, const float* w, cons
     int kw = 1;
     while (kw < 8 && nK > 4 * kw) kw *= 2;
     const int nPT16 = ceil_div(P, 16), nOT16 = ceil_div(O, 16);
-    launch(conv1x1_mfma16_kernel<true>, dim3(nPT16 * nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
-           in, w, bias, out, P, I, O, nPT16, relu, Win, Hin, Wp);
+    DRHIP_REQUIRE(nOT16 <= 65535, "drhip_conv1x1_pooled3s2_f32: too many output channels (%d)", O);
+    launch(conv1x1_mfma16_kernel<true>, dim3(nPT16, nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
+           in, w, bias, out, P, I, O, nPT16, relu, Win, Hin, make_fastdiv(Wp));
     return launched("conv1x1_mfma16_kernel<pooled input>");
 }

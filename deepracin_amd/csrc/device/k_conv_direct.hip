@@ -41,8 +41,8 @@ conv_direct_kernel(const float* __restrict__ in, const float* __restrict__ w, co
     float* filt = lds + CC * patchN;            // [CC][taps][OCT]
 
     const int tid = threadIdx.x, tx = tid % kDirTile, ty = tid / kDirTile;
-    const int tileX = blockIdx.x % tilesX, tileY = blockIdx.x / tilesX;
-    const int o0 = blockIdx.y * OCT;
+    const int tileX = blockIdx.x, tileY = blockIdx.y;       // (a 3-D grid: no integer division in front of the first loads)
+    const int o0 = blockIdx.z * OCT;
     const int xo = tileX * kDirTile + tx, yo = tileY * kDirTile + ty;
     const int px0 = tileX * kDirTile * sx - kw / 2, py0 = tileY * kDirTile * sy - kh / 2;
 
@@ -117,8 +117,8 @@ conv_direct_fewc_kernel(const float* __restrict__ in, const float* __restrict__ 
                         int sx, int sy, int tilesX, int relu) {
     constexpr int taps = KW * KH;
     const int tid = threadIdx.x, tx = tid % kDirTile, ty = tid / kDirTile;
-    const int tileX = blockIdx.x % tilesX, tileY = blockIdx.x / tilesX;
-    const int o0 = blockIdx.y * OCT;
+    const int tileX = blockIdx.x, tileY = blockIdx.y;       // (a 3-D grid: no integer division in front of the first loads)
+    const int o0 = blockIdx.z * OCT;
     const int xo = tileX * kDirTile + tx, yo = tileY * kDirTile + ty;
     const int cx = min(xo, Wo - 1) * sx - KW / 2, cy = min(yo, Ho - 1) * sy - KH / 2;   // window origin (clamped lanes recompute a valid pixel)
 
@@ -192,8 +192,8 @@ conv3x3_fewc_pool3s2_kernel(const float* __restrict__ in, const float* __restric
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 15, lk = lane >> 4;
-    const int tileX = blockIdx.x % tilesX, tileY = blockIdx.x / tilesX;
-    const int o0 = blockIdx.y * 16 * MB;
+    const int tileX = blockIdx.x, tileY = blockIdx.y;       // (a 3-D grid: no integer division in front of the first loads)
+    const int o0 = blockIdx.z * 16 * MB;
 
     const int q = 16 * wave + j;                    // convolution pixel within the 9x9 tile
     const int ry = q / kFpConv, rx = q % kFpConv;
@@ -296,8 +296,8 @@ conv3x3_fewc_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 15, lk = lane >> 4;
-    const int tileX = blockIdx.x % tilesX, tileY = blockIdx.x / tilesX;
-    const int o0 = blockIdx.y * OBc;
+    const int tileX = blockIdx.x, tileY = blockIdx.y;       // (a 3-D grid: no integer division in front of the first loads)
+    const int o0 = blockIdx.z * OBc;
     const int x = tileX * 16 + j, y = tileY * 4 + wave;
     const bool pixOk = x < Wo && y < Ho;
 
@@ -408,8 +408,9 @@ __device__ inline f32x4d dm_buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset
 template <int NT, int S>                    // 32*NT output channels per workgroup; stride (both directions) 1 or 2
 __global__ void __launch_bounds__(512)
 conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict__ F, const float* __restrict__ bias,
-                           float* __restrict__ out, int W, int H, int I, int O, int Wo, int Ho, int nPT, int relu) {
+                           float* __restrict__ out, int W, int H, int I, int O, FastDiv Wod, int Ho, int nPT, int relu) {
     constexpr int OB = 32 * NT, KC = kDmKC;
+    const int Wo = (int)Wod.d;
     constexpr int NA = NT == 1 ? 2 : 1;     // accumulators per channel block: two independent MFMA chains at least
     extern __shared__ float part[];         // [KW][OB][kDmPartPitch]
 
@@ -417,7 +418,7 @@ conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int KW = blockDim.x >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
-    const int o0 = (blockIdx.x / nPT) * OB, p0 = (blockIdx.x % nPT) * 32;
+    const int o0 = blockIdx.y * OB, p0 = blockIdx.x * 32;
     const int P = Wo * Ho, plane = H * W;
     const int nChunks = (I + KC - 1) / KC, Opad = dm_opad(O);
 
@@ -425,7 +426,7 @@ conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict
     const int p = p0 + l32;
     const bool pOk = p < P;
     const int pc = min(p, P - 1);
-    const int y = pc / Wo, x = pc - y * Wo;
+    const int y = fast_div(pc, Wod), x = pc - y * Wo;
     // The window starts at column x*S - 1.  Only x = 0 starts left of the image: that lane loads from column 0
     // and shifts its samples up by one (a negative offset would zero the whole load for the first pixel).
     const bool shifted = x == 0;
@@ -571,7 +572,8 @@ static int launch_direct(const float* in, const float* w, const float* bias, flo
     if (CC > I) CC = I;
     DRHIP_REQUIRE(CC >= 1, "drhip_conv2d_direct_f32: a %dx%d filter with stride %dx%d does not fit the LDS patch", kw, kh, sx, sy);
     const size_t ldsBytes = (size_t)CC * perChannel * sizeof(float);
-    dim3 grid(tilesX * tilesY, ceil_div(O, OCT)), block(kDirThreads);
+    if (tilesY > 65535 || ceil_div(O, OCT) > 65535) return fail(DRHIP_EINVAL, "drhip_conv2d_direct_f32: %d rows of tiles x %d channel blocks exceed the launch grid", tilesY, ceil_div(O, OCT));
+    dim3 grid(tilesX, tilesY, ceil_div(O, OCT)), block(kDirThreads);
     if (kw == 3 && kh == 3)
         launch((conv_direct_kernel<OCT, 3, 3>), grid, block, ldsBytes, s, in, w, bias, out, W, H, I, O, Wo, Ho, kw, kh, sx, sy, CC, tilesX, relu);
     else
@@ -602,7 +604,8 @@ extern "C" int drhip_conv2d_direct_f32(const float* in, const float* w, const fl
         const int tilesX = ceil_div(Wo, 16), tilesY = ceil_div(Ho, 4);
         const int ks = ceil_div(9 * I, 4);
         const bool wide = O > 32;
-        const dim3 grid(tilesX * tilesY, ceil_div(O, wide ? 64 : 32)), block(256);
+        DRHIP_REQUIRE(tilesY <= 65535 && O <= 32 * 65535, "drhip_conv2d_direct_f32: tensor exceeds the launch grid");
+        const dim3 grid(tilesX, tilesY, ceil_div(O, wide ? 64 : 32)), block(256);
 #define DRHIP_FM(MBV, KSV) launch((conv3x3_fewc_mfma_kernel<MBV, KSV>), grid, block, 0, s0, in, w, bias, out, W, H, I, O, Wo, Ho, strideX, strideY, tilesX, relu)
 #define DRHIP_FM_K(MBV) do { if (ks == 3) DRHIP_FM(MBV, 3); else if (ks == 5) DRHIP_FM(MBV, 5); else if (ks == 7) DRHIP_FM(MBV, 7); else DRHIP_FM(MBV, 9); } while (0)
         if (wide) DRHIP_FM_K(4); else DRHIP_FM_K(2);
@@ -613,7 +616,8 @@ extern "C" int drhip_conv2d_direct_f32(const float* in, const float* w, const fl
     if (I <= 4 && kw == 3 && kh == 3) {
         const int Wo = W / strideX, Ho = H / strideY;
         const int tilesX = ceil_div(Wo, kDirTile), tilesY = ceil_div(Ho, kDirTile);
-#define DRHIP_FEWC(OCTV, ICV) launch((conv_direct_fewc_kernel<OCTV, 3, 3, ICV>), dim3(tilesX * tilesY, ceil_div(O, OCTV)), dim3(kDirThreads), 0, s0, \
+        DRHIP_REQUIRE(tilesY <= 65535 && O <= 65535, "drhip_conv2d_direct_f32: tensor exceeds the launch grid");
+#define DRHIP_FEWC(OCTV, ICV) launch((conv_direct_fewc_kernel<OCTV, 3, 3, ICV>), dim3(tilesX, tilesY, ceil_div(O, OCTV)), dim3(kDirThreads), 0, s0, \
                                      in, w, bias, out, W, H, I, O, Wo, Ho, strideX, strideY, tilesX, relu)
 #define DRHIP_FEWC_I(OCTV) do { if (I == 1) DRHIP_FEWC(OCTV, 1); else if (I == 2) DRHIP_FEWC(OCTV, 2); else if (I == 3) DRHIP_FEWC(OCTV, 3); else DRHIP_FEWC(OCTV, 4); } while (0)
         if (O >= 8) DRHIP_FEWC_I(8);            // 16 channels per lane measured slower (8.0 vs 6.6 us on 224x224x3 -> 64)
@@ -643,7 +647,8 @@ extern "C" int drhip_conv3x3_pool3s2_f32(const float* in, const float* w, const 
     hipStream_t s = as_stream(stream);
     const int ks = ceil_div(9 * I, 4);              // 3, 5, 7 or 9
     const bool wide = O > 32;                       // 64 channels per workgroup, else 32
-    const dim3 grid(tilesX * tilesY, ceil_div(O, wide ? 64 : 32)), block(kFpThreads);
+    DRHIP_REQUIRE(tilesY <= 65535 && O <= 32 * 65535, "drhip_conv3x3_pool3s2_f32: tensor exceeds the launch grid");
+    const dim3 grid(tilesX, tilesY, ceil_div(O, wide ? 64 : 32)), block(kFpThreads);
 #define DRHIP_FP(MBV, KSV) launch((conv3x3_fewc_pool3s2_kernel<MBV, KSV>), grid, block, 0, s, in, w, bias, out, W, H, I, O, Wo, Ho, Wp, Hp, strideX, strideY, tilesX, relu)
 #define DRHIP_FP_K(MBV) do { if (ks == 3) DRHIP_FP(MBV, 3); else if (ks == 5) DRHIP_FP(MBV, 5); else if (ks == 7) DRHIP_FP(MBV, 7); else DRHIP_FP(MBV, 9); } while (0)
     if (wide) DRHIP_FP_K(4); else DRHIP_FP_K(2);
@@ -696,10 +701,11 @@ extern "C" int drhip_conv3x3_direct_mfma_f32(const float* in, const float* F, co
     DRHIP_REQUIRE((variant >> 5) == 0 && (kw == 1 || kw == 2 || kw == 4 || kw == 8), "drhip_conv3x3_direct_mfma_f32: unknown variant %#x", variant);
     const int OB = wide ? 64 : 32;
     const int nPT = ceil_div(Wo * Ho, 32);
-    const dim3 grid(nPT * ceil_div(O, OB)), block(64 * kw);
+    DRHIP_REQUIRE(ceil_div(O, OB) <= 65535, "drhip_conv3x3_direct_mfma_f32: too many output channels (%d)", O);
+    const dim3 grid(nPT, ceil_div(O, OB)), block(64 * kw);
     const size_t ldsBytes = (size_t)kw * OB * kDmPartPitch * sizeof(float);
     hipStream_t s = as_stream(stream);
-#define DRHIP_DM(NTV, SV) launch((conv3x3_direct_mfma_kernel<NTV, SV>), grid, block, ldsBytes, s, in, F, bias, out, W, H, I, O, Wo, Ho, nPT, relu)
+#define DRHIP_DM(NTV, SV) launch((conv3x3_direct_mfma_kernel<NTV, SV>), grid, block, ldsBytes, s, in, F, bias, out, W, H, I, O, make_fastdiv(Wo), Ho, nPT, relu)
     if (wide) { if (stride == 1) DRHIP_DM(2, 1); else DRHIP_DM(2, 2); }
     else { if (stride == 1) DRHIP_DM(1, 1); else DRHIP_DM(1, 2); }
 #undef DRHIP_DM

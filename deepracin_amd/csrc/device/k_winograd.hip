@@ -159,17 +159,19 @@ template <int NT, int KW>
 __global__ void __launch_bounds__(kWinoThreads * KW, KW == 2 ? 1 : (NT == 1 ? 3 : (NT == 2 ? 2 : 1)))
 winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__ U,
                          const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
-                         int W, int H, int I, int O, int tilesX, int T, int nTB, int nBlocks,
+                         int W, int H, int I, int O, FastDiv tilesXd, int T, FastDiv nTBd, int nBlocks,
                          int chunksPerSplit, int relu, int vec2) {
     constexpr int TB = 32, OB = 32 * NT, KC = kWinoKC;
+    const int tilesX = (int)tilesXd.d;
     extern __shared__ float P[];                    // epilogue only: [KW sets][4 rows][2][OB o][32 t] floats
 
     // ---- which panel: XCD-aware remap of the linear workgroup id -----------------------------
     const int perXcd = gridDim.x / kXcds;           // grid is padded to a multiple of kXcds
     const int logical = (blockIdx.x % kXcds) * perXcd + blockIdx.x / kXcds;
     if (logical >= nBlocks) return;
-    const int o0 = (logical / nTB) * OB;
-    const int t0 = (logical % nTB) * TB;
+    const int oBlock = fast_div(logical, nTBd);
+    const int o0 = oBlock * OB;
+    const int t0 = (logical - oBlock * (int)nTBd.d) * TB;
     const int split = blockIdx.y, nSplits = gridDim.y;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -187,7 +189,7 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     // Row w of B^T d:  w=0: d0 - d2,  w=1: d1 + d2,  w=2: d2 - d1,  w=3: d3 - d1.
     const int tg = t0 + l32;
     const bool tileOk = tg < T;
-    const int ty = tileOk ? tg / tilesX : 0, tx = tileOk ? tg % tilesX : 0;
+    const int ty = tileOk ? fast_div(tg, tilesXd) : 0, tx = tileOk ? tg - ty * tilesX : 0;
     const int x0 = 2 * tx - 1, y0 = 2 * ty - 1;
     const int rowA = wave, rowB = (wave < 2) ? 2 : 1;
     const float sgn = (wave == 1) ? 1.0f : -1.0f;
@@ -336,7 +338,8 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     const int et = tid & 31, eo = tid >> 5;
     const int etg = t0 + et;
     const bool eTileOk = etg < T;
-    const int ox = eTileOk ? 2 * (etg % tilesX) : 0, oy = eTileOk ? 2 * (etg / tilesX) : 0;
+    const int eTy = eTileOk ? fast_div(etg, tilesXd) : 0;
+    const int ox = eTileOk ? 2 * (etg - eTy * tilesX) : 0, oy = 2 * eTy;
     f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
 #pragma unroll
     for (int q = 0; q < OB / EO; ++q) {
@@ -387,16 +390,18 @@ template <int NB, int KW>
 __global__ void __launch_bounds__(kWinoThreads * KW)
 winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ U,
                            const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
-                           int W, int H, int I, int O, int tilesX, int T, int nTB, int nBlocks,
+                           int W, int H, int I, int O, FastDiv tilesXd, int T, FastDiv nTBd, int nBlocks,
                            int chunksPerSplit, int relu, int vec2) {
     constexpr int TB = 16, OB = 16 * NB, KC = kWinoKC;
+    const int tilesX = (int)tilesXd.d;
     extern __shared__ float P[];                    // epilogue only: [KW sets][4 rows][2][OB o][16 t] floats
 
     const int perXcd = gridDim.x / kXcds;
     const int logical = (blockIdx.x % kXcds) * perXcd + blockIdx.x / kXcds;
     if (logical >= nBlocks) return;
-    const int o0 = (logical / nTB) * OB;
-    const int t0 = (logical % nTB) * TB;
+    const int oBlock = fast_div(logical, nTBd);
+    const int o0 = oBlock * OB;
+    const int t0 = (logical - oBlock * (int)nTBd.d) * TB;
     const int split = blockIdx.y, nSplits = gridDim.y;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -413,7 +418,7 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
     // window rows, offsets and edge masks exactly as in the 32-tile kernel
     const int tg = t0 + l16;
     const bool tileOk = tg < T;
-    const int ty = tileOk ? tg / tilesX : 0, tx = tileOk ? tg % tilesX : 0;
+    const int ty = tileOk ? fast_div(tg, tilesXd) : 0, tx = tileOk ? tg - ty * tilesX : 0;
     const int x0 = 2 * tx - 1, y0 = 2 * ty - 1;
     const int rowA = wave, rowB = (wave < 2) ? 2 : 1;
     const float sgn = (wave == 1) ? 1.0f : -1.0f;
@@ -534,7 +539,8 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
     const int et = tid & 15, eo = tid >> 4;
     const int etg = t0 + et;
     const bool eTileOk = etg < T;
-    const int ox = eTileOk ? 2 * (etg % tilesX) : 0, oy = eTileOk ? 2 * (etg / tilesX) : 0;
+    const int eTy = eTileOk ? fast_div(etg, tilesXd) : 0;
+    const int ox = eTileOk ? 2 * (etg - eTy * tilesX) : 0, oy = 2 * eTy;
     f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
@@ -575,15 +581,17 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
 // panel's partial tiles a moment ago: they are still in that XCD's L2.
 __global__ void __launch_bounds__(256)
 winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restrict__ bias, float* __restrict__ out,
-                             int W, int H, int O, int tilesX, int T, int nTB, int nBlocks, int perXcd, int TB, int OB,
+                             int W, int H, int O, FastDiv tilesXd, int T, FastDiv nTBd, int nBlocks, int perXcd, int lgTB, int lgOB,
                              int nSplits, int relu, int vec2) {
-    const int blocksPerPanel = (TB * OB) / 256;
-    const int j = blockIdx.x / kXcds;
-    const int panel = (blockIdx.x % kXcds) * perXcd + j / blocksPerPanel;
-    if (j / blocksPerPanel >= perXcd || panel >= nBlocks) return;
-    const int within = (j % blocksPerPanel) * 256 + threadIdx.x;    // (o in panel) * TB + tile in panel
-    const int tLocal = within % TB, ol = within / TB;
-    const int o = (panel / nTB) * OB + ol, tg = (panel % nTB) * TB + tLocal;
+    // (TB, OB and TB * OB / 256 are powers of two: shifts and masks instead of integer divisions)
+    const int TB = 1 << lgTB, OB = 1 << lgOB, lgBpp = lgTB + lgOB - 8;
+    const int j = blockIdx.x / kXcds, jp = j >> lgBpp;
+    const int panel = (blockIdx.x % kXcds) * perXcd + jp;
+    if (jp >= perXcd || panel >= nBlocks) return;
+    const int within = ((j & ((1 << lgBpp) - 1)) << 8) + threadIdx.x;     // (o in panel) * TB + tile in panel
+    const int tLocal = within & (TB - 1), ol = within >> lgTB;
+    const int oBlock = fast_div(panel, nTBd);
+    const int o = oBlock * OB + ol, tg = (panel - oBlock * (int)nTBd.d) * TB + tLocal;
     if (o >= O || tg >= T) return;
     const size_t idx = (size_t)panel * TB * OB + within;
     const f32x4* p = (const f32x4*)ws + idx;
@@ -600,7 +608,8 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
     for (; sp < nSplits; ++sp) s += p[(size_t)sp * splitStride];
     if (bias) s += bias[o];
     if (relu & kEpiRelu) { s[0] = fmaxf(s[0], 0.f); s[1] = fmaxf(s[1], 0.f); s[2] = fmaxf(s[2], 0.f); s[3] = fmaxf(s[3], 0.f); }
-    const int ox = 2 * (tg % tilesX), oy = 2 * (tg / tilesX);
+    const int ty = fast_div(tg, tilesXd);
+    const int ox = 2 * (tg - ty * (int)tilesXd.d), oy = 2 * ty;
     if (relu & kEpiMaxPool2)
         store1_through(out + (size_t)o * ((H >> 1) * (W >> 1)) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
     else
@@ -672,22 +681,22 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
             }
             if (c.waveSets == 2)
                 launch((winograd_f23_mfma_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
-                       in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
+                       in, U, bias, out, workspace, W, H, I, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, g.chunksPerSplit, relu, vec2);
         }
         if (c.waveSets != 2 || NT > 2)
             launch((winograd_f23_mfma_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
-                   in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
+                   in, U, bias, out, workspace, W, H, I, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, g.chunksPerSplit, relu, vec2);
     } else if (c.waveSets == 2)
         launch((winograd_f23_mfma16_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
-               in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
+               in, U, bias, out, workspace, W, H, I, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, g.chunksPerSplit, relu, vec2);
     else
         launch((winograd_f23_mfma16_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
-               in, U, bias, out, workspace, W, H, I, O, g.tilesX, g.T, g.nTB, g.nBlocks, g.chunksPerSplit, relu, vec2);
+               in, U, bias, out, workspace, W, H, I, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, g.chunksPerSplit, relu, vec2);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
     if (g.splits > 1) {
         const int perXcd = gridX / kXcds;
         launch(winograd_split_reduce_kernel, dim3(gridX * (OB * TB / 256)), dim3(256), 0, s,
-               workspace, bias, out, W, H, O, g.tilesX, g.T, g.nTB, g.nBlocks, perXcd, TB, OB, g.splits, relu, vec2);
+               workspace, bias, out, W, H, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, perXcd, __builtin_ctz(TB), __builtin_ctz(OB), g.splits, relu, vec2);
         return launched("winograd_split_reduce_kernel");
     }
     return DRHIP_OK;
