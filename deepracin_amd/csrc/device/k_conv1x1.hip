@@ -35,11 +35,12 @@ constexpr int kC1Pad = 33;          // LDS row pitch of a partial tile (floats)
 
 __global__ void __launch_bounds__(512)
 conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
-                    float* __restrict__ out, float* __restrict__ poolPartials, int P, int I, int O, int nPT, int relu) {
+                    float* __restrict__ out, float* __restrict__ poolPartials, int P, int I, int O, int KW, int relu) {
     extern __shared__ float part[];                 // [KW][32][kC1Pad], used only when KW > 1
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int KW = blockDim.x >> 6;
+    // (KW, the waves per workgroup, is a kernel argument: blockDim.x would be a load from the dispatch packet in
+    // front of everything else; the 15 dwords of arguments arrive in SGPRs with the wave)
     const int l32 = lane & 31, lhi = lane >> 5;
     const int o0 = blockIdx.y * 32, p0 = blockIdx.x * 32;      // (a 2-D grid: an integer division here delays the first loads)
     const int nStages = (I + kC1KC - 1) / kC1KC;
@@ -49,7 +50,7 @@ conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, c
     float biasEarly[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-        const int idx = tid + q * (int)blockDim.x;
+        const int idx = tid + q * (64 * KW);
         biasEarly[q] = (bias && idx < 32 * 32) ? bias[min(o0 + (idx >> 5), O - 1)] : 0.0f;
     }
 
@@ -110,7 +111,7 @@ conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, c
     __syncthreads();
 #pragma unroll
     for (int q = 0; q < 8; ++q) {                   // KW >= 2 waves: at most 8 elements per thread
-        const int idx = tid + q * (int)blockDim.x;
+        const int idx = tid + q * (64 * KW);
         if (idx >= 32 * 32) break;
         const int ol = idx >> 5, pl = idx & 31;
         const int o = o0 + ol, p = p0 + pl;
@@ -155,13 +156,16 @@ constexpr unsigned kC1BufferFlags = 0x00020000u;    // dword 3 of a gfx9 raw buf
 template <bool POOL>
 __global__ void __launch_bounds__(POOL ? 512 : 1024)
 conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
-                      float* __restrict__ out, int P, int I, int O, int nPT, int relu, int Win, int Hin, FastDiv Wpd) {
+                      float* __restrict__ out, int P, int I, int O, int KW, int reluAndShift, int Win, int Hin, unsigned WpMul) {
     extern __shared__ float part[];                 // [KW][16][kC1Pad16]
+    const int relu = reluAndShift & 1;              // (16 dwords of arguments in all: they arrive in SGPRs with the wave)
+    const FastDiv Wpd = {(unsigned)((Win + 1) >> 1), WpMul, (unsigned)(reluAndShift >> 8)};
     constexpr int CH = POOL ? 4 : kC1Chunk;         // k-steps per chunk
     constexpr int NS = POOL ? 12 : 1;               // floats loaded per B operand (3 window rows of 4)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int KW = blockDim.x >> 6;
+    // (KW, the waves per workgroup, is a kernel argument: (64 * KW) would be a load from the dispatch packet
+    // in front of everything else)
     const int l16 = lane & 15, lk = lane >> 4;
     const int o0 = blockIdx.y * 16, p0 = blockIdx.x * 16;    // (a 2-D grid: an integer division here delays the first loads)
     const int nK = (I + 3) / 4;                     // k-steps of 4 channels
@@ -186,12 +190,12 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
     }
 
     // The epilogue's bias values are requested now: a load issued there would add a trip to memory to the tail of
-    // every workgroup.  Thread tid finishes the elements tid, tid + blockDim.x, ... of the 16x16 tile (at most 4).
+    // every workgroup.  Thread tid finishes the elements tid, tid + (64 * KW), ... of the 16x16 tile (at most 4).
     float biasEarly[4] = {0.f, 0.f, 0.f, 0.f};
     if (bias) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int idx = tid + q * (int)blockDim.x;
+            const int idx = tid + q * (64 * KW);
             if (idx < 256) biasEarly[q] = bias[min(o0 + (idx >> 4), O - 1)];
         }
     }
@@ -250,7 +254,7 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
     __syncthreads();
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        const int idx = tid + q * (int)blockDim.x;
+        const int idx = tid + q * (64 * KW);
         if (idx >= 16 * 16) break;
         const int ol = idx >> 4, pl = idx & 15;
         const int o = o0 + ol, p = p0 + pl;
@@ -301,7 +305,7 @@ extern "C" int drhip_conv1x1_f32(const float* in, const float* w, const float* b
         const int nPT16 = ceil_div(P, 16), nOT16 = ceil_div(O, 16);
         DRHIP_REQUIRE(nOT16 <= 65535, "drhip_conv1x1_f32: too many output channels for 16x16 tiles (%d)", O);
         launch(conv1x1_mfma16_kernel<false>, dim3(nPT16, nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
-               in, w, bias, out, P, I, O, nPT16, relu, 0, 0, make_fastdiv(1));
+               in, w, bias, out, P, I, O, kw, relu ? 1 : 0, 0, 0, 0u);
         return launched("conv1x1_mfma16_kernel");
     }
     DRHIP_REQUIRE(variant == 1 || variant == 2 || variant == 4 || variant == 8, "drhip_conv1x1_f32: unknown variant %d (waves per tile: 1, 2, 4, 8)", variant);
@@ -309,7 +313,7 @@ extern "C" int drhip_conv1x1_f32(const float* in, const float* w, const float* b
     DRHIP_REQUIRE(nOT <= 65535, "drhip_conv1x1_f32: too many output channels (%d)", O);
     const size_t ldsBytes = variant > 1 ? (size_t)variant * 32 * kC1Pad * sizeof(float) : 0;
     launch(conv1x1_mfma_kernel, dim3(nPT, nOT), dim3(64 * variant), ldsBytes, as_stream(stream),
-                       in, w, bias, out, (float*)nullptr, P, I, O, nPT, relu);
+                       in, w, bias, out, (float*)nullptr, P, I, O, variant, relu);
     return launched("conv1x1_mfma_kernel");
 }
 
@@ -328,7 +332,7 @@ extern "C" int drhip_conv1x1_poolsum_f32(const float* in, const float* w, const 
     const int nPT = ceil_div(P, 32), nOT = ceil_div(O, 32);
     DRHIP_REQUIRE(nOT <= 65535, "drhip_conv1x1_poolsum_f32: too many output channels (%d)", O);
     launch(conv1x1_mfma_kernel, dim3(nPT, nOT), dim3(64 * kw), (size_t)kw * 32 * kC1Pad * sizeof(float), as_stream(stream),
-           in, w, bias, (float*)nullptr, partials, P, I, O, nPT, relu);
+           in, w, bias, (float*)nullptr, partials, P, I, O, kw, relu);
     return launched("conv1x1_mfma_kernel");
 }
 
@@ -345,7 +349,8 @@ extern "C" int drhip_conv1x1_pooled3s2_f32(const float* in, const float* w, cons
     while (kw < 8 && nK > 4 * kw) kw *= 2;
     const int nPT16 = ceil_div(P, 16), nOT16 = ceil_div(O, 16);
     DRHIP_REQUIRE(nOT16 <= 65535, "drhip_conv1x1_pooled3s2_f32: too many output channels (%d)", O);
+    const FastDiv dWp = make_fastdiv(Wp);
     launch(conv1x1_mfma16_kernel<true>, dim3(nPT16, nOT16), dim3(64 * kw), (size_t)kw * 16 * kC1Pad16 * sizeof(float), as_stream(stream),
-           in, w, bias, out, P, I, O, nPT16, relu, Win, Hin, make_fastdiv(Wp));
+           in, w, bias, out, P, I, O, kw, (relu ? 1 : 0) | (int)(dWp.shift << 8), Win, Hin, dWp.mul);
     return launched("conv1x1_mfma16_kernel<pooled input>");
 }

@@ -184,8 +184,12 @@ typedef float f32x4d __attribute__((ext_vector_type(4)));
 template <int MB, int KS>                           // KS = k-steps = ceil(9*I / 4)
 __global__ void __launch_bounds__(kFpThreads)
 conv3x3_fewc_pool3s2_kernel(const float* __restrict__ in, const float* __restrict__ w, const float* __restrict__ bias,
-                            float* __restrict__ out, int W, int H, int I, int O, int Wo, int Ho, int Wp, int Hp,
-                            int sx, int sy, int tilesX, int relu) {
+                            float* __restrict__ out, unsigned wh, unsigned io, unsigned woho, unsigned cfg) {
+    // (12 dwords of arguments, which arrive in SGPRs with the wave: wh = W | H << 16, io = I | O << 16,
+    // woho = Wo | Ho << 16, cfg = sx | sy << 4 | relu << 8)
+    const int W = (int)(wh & 0xffffu), H = (int)(wh >> 16), I = (int)(io & 0xffffu), O = (int)(io >> 16);
+    const int Wo = (int)(woho & 0xffffu), Ho = (int)(woho >> 16), Wp = (Wo + 1) >> 1, Hp = (Ho + 1) >> 1;
+    const int sx = (int)(cfg & 15u), sy = (int)((cfg >> 4) & 15u), relu = (int)((cfg >> 8) & 1u);
     __shared__ float convT[16 * MB * kFpPitch];
     __shared__ float wT[4 * KS * 16 * MB];          // filters as [k = (channel, tap)][channel out], zero padded
     __shared__ float biasT[16 * MB];
@@ -408,15 +412,21 @@ __device__ inline f32x4d dm_buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset
 template <int NT, int S>                    // 32*NT output channels per workgroup; stride (both directions) 1 or 2
 __global__ void __launch_bounds__(512)
 conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict__ F, const float* __restrict__ bias,
-                           float* __restrict__ out, int W, int H, int I, int O, FastDiv Wod, int Ho, int nPT, int relu) {
+                           float* __restrict__ out, unsigned wh, unsigned io, unsigned WoMul, unsigned cfg) {
+    // 12 dwords of arguments, all of which arrive in SGPRs with the wave (nothing is read from the dispatch packet:
+    // a scalar load in front of the first vector loads is a round trip of its own in every workgroup):
+    // wh = W | H << 16, io = I | O << 16, WoMul / cfg & 31 = multiplier / shift of the division by Wo,
+    // cfg bit 5 = ReLU, cfg >> 8 = waves per workgroup.
     constexpr int OB = 32 * NT, KC = kDmKC;
-    const int Wo = (int)Wod.d;
+    const int W = (int)(wh & 0xffffu), H = (int)(wh >> 16), I = (int)(io & 0xffffu), O = (int)(io >> 16);
+    const int Wo = W / S, Ho = H / S;
+    const FastDiv Wod = {(unsigned)Wo, WoMul, cfg & 31u};
+    const int relu = (int)((cfg >> 5) & 1u), KW = (int)(cfg >> 8);
     constexpr int NA = NT == 1 ? 2 : 1;     // accumulators per channel block: two independent MFMA chains at least
     extern __shared__ float part[];         // [KW][OB][kDmPartPitch]
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int KW = blockDim.x >> 6;
     const int l32 = lane & 31, lhi = lane >> 5;
     const int o0 = blockIdx.y * OB, p0 = blockIdx.x * 32;
     const int P = Wo * Ho, plane = H * W;
@@ -472,7 +482,7 @@ conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict
     float biasEarly[kMaxEpi];
 #pragma unroll
     for (int q = 0; q < kMaxEpi; ++q) {
-        const int idx = tid + q * (int)blockDim.x;
+        const int idx = tid + q * (64 * KW);
         biasEarly[q] = (bias && idx < OB * 32) ? bias[min(o0 + (idx >> 5), O - 1)] : 0.0f;
     }
 
@@ -553,10 +563,10 @@ conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict
     };
 #pragma unroll
     for (int q = 0; q < kMaxEpi; ++q) {
-        const int idx = tid + q * (int)blockDim.x;
+        const int idx = tid + q * (64 * KW);
         if (idx < OB * 32) finish(idx, biasEarly[q]);
     }
-    for (int idx = tid + kMaxEpi * (int)blockDim.x; idx < OB * 32; idx += blockDim.x)      // one wave per workgroup only
+    for (int idx = tid + kMaxEpi * (64 * KW); idx < OB * 32; idx += 64 * KW)      // one wave per workgroup only
         finish(idx, bias ? bias[min(o0 + (idx >> 5), O - 1)] : 0.0f);
 }
 
@@ -642,6 +652,7 @@ extern "C" int drhip_conv3x3_pool3s2_f32(const float* in, const float* w, const 
     DRHIP_REQUIRE(W > 0 && H > 0 && O > 0 && I >= 1 && I <= 4, "drhip_conv3x3_pool3s2_f32: bad shape %dx%dx%d -> %d (1 to 4 input channels)", W, H, I, O);
     DRHIP_REQUIRE(strideX > 0 && strideY > 0 && W / strideX > 0 && H / strideY > 0, "drhip_conv3x3_pool3s2_f32: bad stride or empty output");
     DRHIP_REQUIRE((long long)W * H * I < (1ll << 31) && (long long)W * H * O < (1ll << 31), "drhip_conv3x3_pool3s2_f32: tensor too large");
+    DRHIP_REQUIRE(W <= 65535 && H <= 65535 && O <= 65535 && strideX <= 15 && strideY <= 15, "drhip_conv3x3_pool3s2_f32: W, H and O are limited to 65535, strides to 15");
     const int Wo = W / strideX, Ho = H / strideY, Wp = ceil_div(Wo, 2), Hp = ceil_div(Ho, 2);
     const int tilesX = ceil_div(Wp, kFpPool), tilesY = ceil_div(Hp, kFpPool);
     hipStream_t s = as_stream(stream);
@@ -649,7 +660,7 @@ extern "C" int drhip_conv3x3_pool3s2_f32(const float* in, const float* w, const 
     const bool wide = O > 32;                       // 64 channels per workgroup, else 32
     DRHIP_REQUIRE(tilesY <= 65535 && O <= 32 * 65535, "drhip_conv3x3_pool3s2_f32: tensor exceeds the launch grid");
     const dim3 grid(tilesX, tilesY, ceil_div(O, wide ? 64 : 32)), block(kFpThreads);
-#define DRHIP_FP(MBV, KSV) launch((conv3x3_fewc_pool3s2_kernel<MBV, KSV>), grid, block, 0, s, in, w, bias, out, W, H, I, O, Wo, Ho, Wp, Hp, strideX, strideY, tilesX, relu)
+#define DRHIP_FP(MBV, KSV) launch((conv3x3_fewc_pool3s2_kernel<MBV, KSV>), grid, block, 0, s, in, w, bias, out, (unsigned)W | (unsigned)H << 16, (unsigned)I | (unsigned)O << 16, (unsigned)Wo | (unsigned)Ho << 16, (unsigned)strideX | (unsigned)strideY << 4 | (relu ? 256u : 0u))
 #define DRHIP_FP_K(MBV) do { if (ks == 3) DRHIP_FP(MBV, 3); else if (ks == 5) DRHIP_FP(MBV, 5); else if (ks == 7) DRHIP_FP(MBV, 7); else DRHIP_FP(MBV, 9); } while (0)
     if (wide) DRHIP_FP_K(4); else DRHIP_FP_K(2);
 #undef DRHIP_FP_K
@@ -690,6 +701,7 @@ extern "C" int drhip_conv3x3_direct_mfma_f32(const float* in, const float* F, co
     DRHIP_REQUIRE(in && F && out, "drhip_conv3x3_direct_mfma_f32: NULL tensor");
     DRHIP_REQUIRE(W > 0 && H > 0 && I > 0 && O > 0, "drhip_conv3x3_direct_mfma_f32: bad shape %dx%dx%d -> %d", W, H, I, O);
     DRHIP_REQUIRE(stride == 1 || stride == 2, "drhip_conv3x3_direct_mfma_f32: stride %d (1 or 2)", stride);
+    DRHIP_REQUIRE(W <= 65535 && H <= 65535 && I <= 65535 && O <= 65535, "drhip_conv3x3_direct_mfma_f32: W, H, I and O are limited to 65535 (got %dx%dx%d -> %d)", W, H, I, O);
     const int Wo = W / stride, Ho = H / stride;
     DRHIP_REQUIRE(Wo > 0 && Ho > 0, "drhip_conv3x3_direct_mfma_f32: output is empty");
     // byte offsets into the input and the filters are 32-bit, and 0x80000000 must lie outside both
@@ -705,7 +717,8 @@ extern "C" int drhip_conv3x3_direct_mfma_f32(const float* in, const float* F, co
     const dim3 grid(nPT, ceil_div(O, OB)), block(64 * kw);
     const size_t ldsBytes = (size_t)kw * OB * kDmPartPitch * sizeof(float);
     hipStream_t s = as_stream(stream);
-#define DRHIP_DM(NTV, SV) launch((conv3x3_direct_mfma_kernel<NTV, SV>), grid, block, ldsBytes, s, in, F, bias, out, W, H, I, O, make_fastdiv(Wo), Ho, nPT, relu)
+    const FastDiv dWo = make_fastdiv(Wo);
+#define DRHIP_DM(NTV, SV) launch((conv3x3_direct_mfma_kernel<NTV, SV>), grid, block, ldsBytes, s, in, F, bias, out, (unsigned)W | (unsigned)H << 16, (unsigned)I | (unsigned)O << 16, dWo.mul, dWo.shift | (relu ? 32u : 0u) | (unsigned)kw << 8)
     if (wide) { if (stride == 1) DRHIP_DM(2, 1); else DRHIP_DM(2, 2); }
     else { if (stride == 1) DRHIP_DM(1, 1); else DRHIP_DM(1, 2); }
 #undef DRHIP_DM

@@ -142,6 +142,23 @@ __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, 
 // gridDim.y = number of input-channel splits KS.  KS == 1: the workgroup finishes its outputs.
 // KS > 1: every split stores its partial (pre-bias) 2x2 tiles, tile-major, to the workspace and
 // winograd_split_reduce_kernel sums them in split order, adds the bias and applies ReLU.
+// The shape arguments of the convolution kernels, packed into six dwords: together with the five pointers they
+// fill exactly the 16 dwords that arrive in SGPRs with the wave (kernel-argument preload).  Everything else is
+// derived; nothing is read from the dispatch packet (gridDim, blockDim), because every scalar load in front of the
+// first vector loads is a round trip of its own at the start of every workgroup (~0.07 us each).
+//   wh = W | H << 16, io = I | O << 16 (each at most 65535),
+//   mulX, mulTB = multipliers of the divisions by tilesX and by the number of tile panels,
+//   cfg0 = shiftX | shiftTB << 5 | epilogue flags << 10 (2 bits) | vec2 << 12 | splits << 13,  cfg1 = chunks per split
+#define WINO_ARGS unsigned wh, unsigned io, unsigned mulX, unsigned mulTB, unsigned cfg0, unsigned cfg1
+#define WINO_UNPACK(TBV, OBV)                                                                           \
+    const int W = (int)(wh & 0xffffu), H = (int)(wh >> 16), I = (int)(io & 0xffffu), O = (int)(io >> 16); \
+    const int tilesX = (W + 1) >> 1, T = tilesX * ((H + 1) >> 1);                                         \
+    const int nTB = (T + (TBV) - 1) / (TBV), nBlocks = nTB * ((O + (OBV) - 1) / (OBV));                   \
+    const FastDiv tilesXd = {(unsigned)tilesX, mulX, cfg0 & 31u}, nTBd = {(unsigned)nTB, mulTB, (cfg0 >> 5) & 31u}; \
+    const int relu = (int)((cfg0 >> 10) & 3u), vec2 = (int)((cfg0 >> 12) & 1u), nSplits = (int)(cfg0 >> 13); \
+    const int chunksPerSplit = (int)cfg1;
+struct WinoPackedArgs { unsigned wh, io, mulX, mulTB, cfg0, cfg1; };
+
 constexpr unsigned kBufferFlags = 0x00020000u;      // dword 3 of a gfx9 raw buffer resource (32-bit data format)
 constexpr int kEpiRelu = DRHIP_EPILOGUE_RELU, kEpiMaxPool2 = DRHIP_EPILOGUE_MAXPOOL2;   // bits of the `relu` argument
 constexpr unsigned kOutOfRange = 0x80000000u;       // byte offset no resource of at most 2 GiB contains
@@ -159,20 +176,19 @@ template <int NT, int KW>
 __global__ void __launch_bounds__(kWinoThreads * KW, KW == 2 ? 1 : (NT == 1 ? 3 : (NT == 2 ? 2 : 1)))
 winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__ U,
                          const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
-                         int W, int H, int I, int O, FastDiv tilesXd, int T, FastDiv nTBd, int nBlocks,
-                         int chunksPerSplit, int relu, int vec2) {
+                         WINO_ARGS) {
     constexpr int TB = 32, OB = 32 * NT, KC = kWinoKC;
-    const int tilesX = (int)tilesXd.d;
+    WINO_UNPACK(TB, OB)
     extern __shared__ float P[];                    // epilogue only: [KW sets][4 rows][2][OB o][32 t] floats
 
     // ---- which panel: XCD-aware remap of the linear workgroup id -----------------------------
-    const int perXcd = gridDim.x / kXcds;           // grid is padded to a multiple of kXcds
+    const int perXcd = (nBlocks + kXcds - 1) / kXcds;   // the grid is padded to a multiple of kXcds
     const int logical = (blockIdx.x % kXcds) * perXcd + blockIdx.x / kXcds;
     if (logical >= nBlocks) return;
     const int oBlock = fast_div(logical, nTBd);
     const int o0 = oBlock * OB;
     const int t0 = (logical - oBlock * (int)nTBd.d) * TB;
-    const int split = blockIdx.y, nSplits = gridDim.y;
+    const int split = blockIdx.y;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int waveId = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -239,7 +255,7 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     constexpr bool kBiasEarly = NT <= 2;
     constexpr int EO = 8 * KW;                      // output channels finished per pass of the epilogue
     float biasEarly[kBiasEarly ? OB / EO : 1];
-    if (kBiasEarly && bias && gridDim.y == 1) {
+    if (kBiasEarly && bias && nSplits == 1) {
 #pragma unroll
         for (int q = 0; q < OB / EO; ++q) biasEarly[q] = bias[min(o0 + (tid >> 5) + EO * q, O - 1)];
     }
@@ -390,19 +406,18 @@ template <int NB, int KW>
 __global__ void __launch_bounds__(kWinoThreads * KW)
 winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ U,
                            const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
-                           int W, int H, int I, int O, FastDiv tilesXd, int T, FastDiv nTBd, int nBlocks,
-                           int chunksPerSplit, int relu, int vec2) {
+                           WINO_ARGS) {
     constexpr int TB = 16, OB = 16 * NB, KC = kWinoKC;
-    const int tilesX = (int)tilesXd.d;
+    WINO_UNPACK(TB, OB)
     extern __shared__ float P[];                    // epilogue only: [KW sets][4 rows][2][OB o][16 t] floats
 
-    const int perXcd = gridDim.x / kXcds;
+    const int perXcd = (nBlocks + kXcds - 1) / kXcds;
     const int logical = (blockIdx.x % kXcds) * perXcd + blockIdx.x / kXcds;
     if (logical >= nBlocks) return;
     const int oBlock = fast_div(logical, nTBd);
     const int o0 = oBlock * OB;
     const int t0 = (logical - oBlock * (int)nTBd.d) * TB;
-    const int split = blockIdx.y, nSplits = gridDim.y;
+    const int split = blockIdx.y;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int waveId = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -454,7 +469,7 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
     constexpr int EO = 16 * KW;                     // output channels finished per pass of the epilogue
     constexpr int NQ = (OB + EO - 1) / EO;
     float biasEarly[NQ];
-    if (bias && gridDim.y == 1) {
+    if (bias && nSplits == 1) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) biasEarly[q] = bias[min(o0 + (tid >> 4) + EO * q, O - 1)];
     }
@@ -580,11 +595,17 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
 // Workgroup b works for panel (b % 8) * perXcd + ..., i.e. on the XCD whose workgroups wrote that
 // panel's partial tiles a moment ago: they are still in that XCD's L2.
 __global__ void __launch_bounds__(256)
-winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restrict__ bias, float* __restrict__ out,
-                             int W, int H, int O, FastDiv tilesXd, int T, FastDiv nTBd, int nBlocks, int perXcd, int lgTB, int lgOB,
-                             int nSplits, int relu, int vec2) {
-    // (TB, OB and TB * OB / 256 are powers of two: shifts and masks instead of integer divisions)
+winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restrict__ bias, float* __restrict__ out, WINO_ARGS) {
+    // (TB, OB and TB * OB / 256 are powers of two: shifts and masks instead of integer divisions; cfg1 carries
+    // log2 TB and log2 OB above the chunk count)
+    const int lgTB = (int)((cfg1 >> 16) & 15u), lgOB = (int)((cfg1 >> 20) & 15u);
     const int TB = 1 << lgTB, OB = 1 << lgOB, lgBpp = lgTB + lgOB - 8;
+    const int W = (int)(wh & 0xffffu), H = (int)(wh >> 16), O = (int)(io >> 16);
+    const int tilesX = (W + 1) >> 1, T = tilesX * ((H + 1) >> 1);
+    const int nTB = (T + TB - 1) >> lgTB, nBlocks = nTB * ((O + OB - 1) >> lgOB);
+    const FastDiv tilesXd = {(unsigned)tilesX, mulX, cfg0 & 31u}, nTBd = {(unsigned)nTB, mulTB, (cfg0 >> 5) & 31u};
+    const int relu = (int)((cfg0 >> 10) & 3u), vec2 = (int)((cfg0 >> 12) & 1u), nSplits = (int)(cfg0 >> 13);
+    const int perXcd = (nBlocks + kXcds - 1) / kXcds;
     const int j = blockIdx.x / kXcds, jp = j >> lgBpp;
     const int panel = (blockIdx.x % kXcds) * perXcd + jp;
     if (jp >= perXcd || panel >= nBlocks) return;
@@ -665,6 +686,10 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
     const int gridX = ceil_div(g.nBlocks, kXcds) * kXcds;
     const size_t ldsBytes = 4 * 2 * OB * TB * sizeof(float);
     const int vec2 = ((W & 1) == 0) && (((size_t)out & 7) == 0);
+    const FastDiv dx = make_fastdiv(g.tilesX), dtb = make_fastdiv(g.nTB);
+    const WinoPackedArgs pa = {(unsigned)W | (unsigned)H << 16, (unsigned)I | (unsigned)O << 16, dx.mul, dtb.mul,
+                               dx.shift | dtb.shift << 5 | (unsigned)(relu & 3) << 10 | (unsigned)vec2 << 12 | (unsigned)g.splits << 13,
+                               (unsigned)g.chunksPerSplit};
     if constexpr (TB == 32) {
         if constexpr (NT <= 2) {
             if (c.waveSets == 2) {
@@ -681,22 +706,22 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
             }
             if (c.waveSets == 2)
                 launch((winograd_f23_mfma_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
-                       in, U, bias, out, workspace, W, H, I, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, g.chunksPerSplit, relu, vec2);
+                       in, U, bias, out, workspace, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1);
         }
         if (c.waveSets != 2 || NT > 2)
             launch((winograd_f23_mfma_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
-                   in, U, bias, out, workspace, W, H, I, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, g.chunksPerSplit, relu, vec2);
+                   in, U, bias, out, workspace, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1);
     } else if (c.waveSets == 2)
         launch((winograd_f23_mfma16_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
-               in, U, bias, out, workspace, W, H, I, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, g.chunksPerSplit, relu, vec2);
+               in, U, bias, out, workspace, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1);
     else
         launch((winograd_f23_mfma16_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
-               in, U, bias, out, workspace, W, H, I, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, g.chunksPerSplit, relu, vec2);
+               in, U, bias, out, workspace, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
     if (g.splits > 1) {
-        const int perXcd = gridX / kXcds;
         launch(winograd_split_reduce_kernel, dim3(gridX * (OB * TB / 256)), dim3(256), 0, s,
-               workspace, bias, out, W, H, O, make_fastdiv(g.tilesX), g.T, make_fastdiv(g.nTB), g.nBlocks, perXcd, __builtin_ctz(TB), __builtin_ctz(OB), g.splits, relu, vec2);
+               workspace, bias, out, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0,
+               pa.cfg1 | (unsigned)__builtin_ctz(TB) << 16 | (unsigned)__builtin_ctz(OB) << 20);
         return launched("winograd_split_reduce_kernel");
     }
     return DRHIP_OK;
@@ -767,6 +792,7 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
     // byte offsets into the input and the filters are 32-bit, and 0x80000000 must lie outside both
     DRHIP_REQUIRE((long long)W * H * I < (1ll << 29) && (long long)W * H * O < (1ll << 31) && (long long)(I + 7) * (O + 31) * 16 < (1ll << 29),
                   "drhip_conv3x3_winograd_f32: tensor too large for 32-bit byte offsets");
+    DRHIP_REQUIRE(W <= 65535 && H <= 65535 && I <= 65535 && O <= 65535, "drhip_conv3x3_winograd_f32: W, H, I and O are limited to 65535 (got %dx%dx%d -> %d)", W, H, I, O);
     DRHIP_REQUIRE(((size_t)U & 15) == 0, "drhip_conv3x3_winograd_f32: transformed filters must be 16-byte aligned");
     DRHIP_REQUIRE((relu & ~(DRHIP_EPILOGUE_RELU | DRHIP_EPILOGUE_MAXPOOL2)) == 0, "drhip_conv3x3_winograd_f32: unknown epilogue flags %d", relu);
     DRHIP_REQUIRE(!(relu & DRHIP_EPILOGUE_MAXPOOL2) || ((W | H) & 1) == 0, "drhip_conv3x3_winograd_f32: the fused 2x2 max pool needs even W and H (got %dx%d)", W, H);

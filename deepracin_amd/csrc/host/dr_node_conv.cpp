@@ -73,6 +73,10 @@ gchar* conv_print(dR_Node* node) {
 gboolean conv_schedule(dR_Graph* net, dR_Node* node) {
     dR_Conv2d_Data* c = conv_of(node);
     const int W = c->ishape.s0, H = c->ishape.s1, I = c->shape.s2, O = c->shape.s3;
+    // The matrix-core convolution kernels carry W, H, I and O in 16-bit fields of their packed arguments;
+    // a layer beyond that takes the general direct kernel.
+    const bool packable = W <= 65535 && H <= 65535 && I <= 65535 && O <= 65535;
+    if (c->algo == drConvWinograd && !packable) c->algo = drConvDirect;
     switch (c->algo) {
         case drConvWinograd: c->variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O); break;
         case drConv1x1Gemm:  c->variant = drhip_conv1x1_pick_variant(W * H, I, O); break;
@@ -80,7 +84,7 @@ gboolean conv_schedule(dR_Graph* net, dR_Node* node) {
             // 3x3, stride 1 or 2, more than 4 input channels: the implicit GEMM on the matrix cores over a filter
             // bank laid out at prepare time; everything else: the direct launcher sizes its own tiles
             const char* valu = getenv("DR_DIRECT_VALU");
-            c->drDirectBank = c->shape.s0 == 3 && c->shape.s1 == 3 && I > 4 && c->stride.s1 == c->stride.s2 &&
+            c->drDirectBank = packable && c->shape.s0 == 3 && c->shape.s1 == 3 && I > 4 && c->stride.s1 == c->stride.s2 &&
                               (c->stride.s1 == 1 || c->stride.s1 == 2) && !(valu && strcmp(valu, "1") == 0);
             c->variant = c->drDirectBank ? drhip_conv3x3_direct_pick_variant(W / c->stride.s1, H / c->stride.s2, I, O) : 0;
             break;

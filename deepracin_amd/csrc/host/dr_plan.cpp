@@ -96,6 +96,8 @@ dR_Node* pool_fusable_producer(const dR_Node* p) {
         if (cd->algo != drConvWinograd || ((c->oshape.s0 | c->oshape.s1) & 1)) return nullptr;
     } else {
         if (cd->algo != drConvDirect || cd->shape.s0 != 3 || cd->shape.s1 != 3 || cd->shape.s2 > 4) return nullptr;
+        // (that kernel carries its shape in 16-bit fields and its strides in 4-bit fields)
+        if (cd->ishape.s0 > 65535 || cd->ishape.s1 > 65535 || cd->shape.s3 > 65535 || cd->stride.s1 > 15 || cd->stride.s2 > 15) return nullptr;
     }
     return c;
 }
