@@ -69,15 +69,18 @@ static FcPlan fc_plan(int K, int N) {
 // wavefronts of the workgroup have rows to stream.
 template <int VEC, bool DEFERRED, int CH>
 __global__ void __launch_bounds__(kFcThreads)
-fc_gemv_kernel(const float* __restrict__ x, drhip_deferred_vec xdef, const float* __restrict__ Wt,
-               const float* __restrict__ bias, float* __restrict__ y, float* __restrict__ partials,
-               int K, int N, int rowsPerSlice, int relu, int defer) {
+fc_gemv_kernel(const float* __restrict__ Wt, const float* __restrict__ x, int K, int N, int rowsPerSlice, int cfg,
+               const float* __restrict__ bias, float* __restrict__ y, float* __restrict__ partials, drhip_deferred_vec xdef) {
+    // The first 14 dwords of arguments arrive in SGPRs with the wave: the matrix, the shape and the output pointers;
+    // the description of a deferred input follows behind them.  cfg = relu | row slices << 8 (the grid's
+    // y extent: read from here, not from the dispatch packet).
+    const int relu = cfg & 1;
     typedef typename VecT<VEC>::type vec_t;
     constexpr int CBW = kWave * VEC;
     __shared__ float red[kFcWaves][CBW];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int panel = blockIdx.x, slice = blockIdx.y, slices = gridDim.y;
+    const int panel = blockIdx.x, slice = blockIdx.y, slices = cfg >> 8;
     // Lanes past the last column re-read the last valid vector (their sums are never stored): the
     // loads stay unconditional, so the compiler can keep a precise count of loads in flight.
     const int col = min(panel * CBW + lane * VEC, N - VEC);
@@ -219,8 +222,10 @@ extern "C" int drhip_fc_slices(int K, int N) {
 template <int VEC, int CH>
 static void launch_gemv_ch(bool deferred, dim3 grid, hipStream_t s, const float* x, const drhip_deferred_vec& xd, const float* Wt,
                            const float* bias, float* y, float* partials, int K, int N, int rowsPerSlice, int relu, int defer) {
-    if (deferred) launch((fc_gemv_kernel<VEC, true, CH>), grid, dim3(kFcThreads), 0, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
-    else launch((fc_gemv_kernel<VEC, false, CH>), grid, dim3(kFcThreads), 0, s, x, xd, Wt, bias, y, partials, K, N, rowsPerSlice, relu, defer);
+    const int cfg = (relu ? 1 : 0) | (int)(grid.y << 8);     // (an unfinished sum is simply one whose finishing kernel is not launched)
+    (void)defer;
+    if (deferred) launch((fc_gemv_kernel<VEC, true, CH>), grid, dim3(kFcThreads), 0, s, Wt, x, K, N, rowsPerSlice, cfg, bias, y, partials, xd);
+    else launch((fc_gemv_kernel<VEC, false, CH>), grid, dim3(kFcThreads), 0, s, Wt, x, K, N, rowsPerSlice, cfg, bias, y, partials, xd);
 }
 
 template <int VEC>

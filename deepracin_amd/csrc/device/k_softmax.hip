@@ -44,7 +44,7 @@ __device__ inline float block_reduce(float v, float* red) {
 // caller wants to read the logits too).
 template <bool SMALL>
 __global__ void __launch_bounds__(kSoftmaxThreads)
-softmax_kernel(const float* x, drhip_deferred_vec xdef, float* y, int n) {     // no __restrict__: x may become y
+softmax_kernel(const float* x, float* y, int n, drhip_deferred_vec xdef) {     // no __restrict__: x may become y
     __shared__ float red[kSoftmaxThreads / kWave];
     const int tid = threadIdx.x;
     if (SMALL) {                                    // n <= kSoftmaxThreads * kSoftmaxRegs
@@ -104,9 +104,9 @@ extern "C" int drhip_softmax_ex_f32(const float* x, const drhip_deferred_vec* xd
     DRHIP_REQUIRE(!xdef || xdef->finished != y, "drhip_softmax_f32: the finished logits and the probabilities need separate arrays");
     const drhip_deferred_vec none = {nullptr, nullptr, 0, 0, 0, nullptr, 0.0f};
     if (n <= kSoftmaxThreads * kSoftmaxRegs)
-        launch(softmax_kernel<true>, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, xdef ? *xdef : none, y, n);
+        launch(softmax_kernel<true>, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, y, n, xdef ? *xdef : none);
     else
-        launch(softmax_kernel<false>, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, xdef ? *xdef : none, y, n);
+        launch(softmax_kernel<false>, dim3(1), dim3(kSoftmaxThreads), 0, as_stream(stream), x, y, n, xdef ? *xdef : none);
     return launched("softmax_kernel");
 }
 

@@ -142,10 +142,12 @@ __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, 
 // gridDim.y = number of input-channel splits KS.  KS == 1: the workgroup finishes its outputs.
 // KS > 1: every split stores its partial (pre-bias) 2x2 tiles, tile-major, to the workspace and
 // winograd_split_reduce_kernel sums them in split order, adds the bias and applies ReLU.
-// The shape arguments of the convolution kernels, packed into six dwords: together with the five pointers they
-// fill exactly the 16 dwords that arrive in SGPRs with the wave (kernel-argument preload).  Everything else is
-// derived; nothing is read from the dispatch packet (gridDim, blockDim), because every scalar load in front of the
-// first vector loads is a round trip of its own at the start of every workgroup (~0.07 us each).
+// The shape arguments of the convolution kernels, packed into six dwords.  The first 14 dwords of a kernel's
+// arguments arrive in SGPRs with the wave (kernel-argument preload: 16 user SGPRs, two of which hold the address
+// of the argument block): the three input pointers, these six dwords and the output pointer; the workspace
+// pointer, which only the epilogue of a split layer needs, comes last.  Everything else is derived; nothing is
+// read from the dispatch packet (gridDim, blockDim), because every scalar load in front of the first vector loads
+// is a round trip of its own at the start of every workgroup (~0.07 us each).
 //   wh = W | H << 16, io = I | O << 16 (each at most 65535),
 //   mulX, mulTB = multipliers of the divisions by tilesX and by the number of tile panels,
 //   cfg0 = shiftX | shiftTB << 5 | epilogue flags << 10 (2 bits) | vec2 << 12 | splits << 13,  cfg1 = chunks per split
@@ -174,9 +176,8 @@ __device__ inline f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset, un
 // without a second workgroup's share of partial tiles in memory.
 template <int NT, int KW>
 __global__ void __launch_bounds__(kWinoThreads * KW, KW == 2 ? 1 : (NT == 1 ? 3 : (NT == 2 ? 2 : 1)))
-winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__ U,
-                         const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
-                         WINO_ARGS) {
+winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__ U, const float* __restrict__ bias,
+                         WINO_ARGS, float* __restrict__ out, float* __restrict__ ws) {
     constexpr int TB = 32, OB = 32 * NT, KC = kWinoKC;
     WINO_UNPACK(TB, OB)
     extern __shared__ float P[];                    // epilogue only: [KW sets][4 rows][2][OB o][32 t] floats
@@ -404,9 +405,8 @@ typedef float f32x4acc __attribute__((ext_vector_type(4)));
 // (14x14, 64 -> 256: 5.1 vs 5.4 us; four sets were measured slower again).
 template <int NB, int KW>
 __global__ void __launch_bounds__(kWinoThreads * KW)
-winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ U,
-                           const float* __restrict__ bias, float* __restrict__ out, float* __restrict__ ws,
-                           WINO_ARGS) {
+winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ U, const float* __restrict__ bias,
+                           WINO_ARGS, float* __restrict__ out, float* __restrict__ ws) {
     constexpr int TB = 16, OB = 16 * NB, KC = kWinoKC;
     WINO_UNPACK(TB, OB)
     extern __shared__ float P[];                    // epilogue only: [KW sets][4 rows][2][OB o][16 t] floats
@@ -706,17 +706,17 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
             }
             if (c.waveSets == 2)
                 launch((winograd_f23_mfma_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
-                       in, U, bias, out, workspace, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1);
+                       in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
         }
         if (c.waveSets != 2 || NT > 2)
             launch((winograd_f23_mfma_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
-                   in, U, bias, out, workspace, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1);
+                   in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
     } else if (c.waveSets == 2)
         launch((winograd_f23_mfma16_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
-               in, U, bias, out, workspace, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1);
+               in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
     else
         launch((winograd_f23_mfma16_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
-               in, U, bias, out, workspace, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1);
+               in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
     if (g.splits > 1) {
         launch(winograd_split_reduce_kernel, dim3(gridX * (OB * TB / 256)), dim3(256), 0, s,
