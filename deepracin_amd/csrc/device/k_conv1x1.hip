@@ -189,17 +189,6 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
         rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kC1BufferFlags);
     }
 
-    // The epilogue's bias values are requested now: a load issued there would add a trip to memory to the tail of
-    // every workgroup.  Thread tid finishes the elements tid, tid + (64 * KW), ... of the 16x16 tile (at most 4).
-    float biasEarly[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int idx = tid + q * (64 * KW);
-            if (idx < 256) biasEarly[q] = bias[min(o0 + (idx >> 4), O - 1)];
-        }
-    }
-
     f32x4v acc = {0.f, 0.f, 0.f, 0.f};
     float aA[CH], bA[CH][NS], aB[CH], bB[CH][NS];
     // chunk j of this wave = its k-steps wave + KW*(CH*j .. CH*j + CH-1)
@@ -240,6 +229,14 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
     // Two buffers, the next chunk always on its way.  The loop leaves right after the last real
     // chunk: the loads issued beyond it (clamped addresses) are never waited for.
     load_chunk(aA, bA, 0);
+    // The epilogue's bias values are requested now, behind the first operands: a load issued in the epilogue would
+    // add a trip to memory to the tail of every workgroup.  Thread tid finishes the elements tid, tid + 64 KW, ...
+    // of the 16x16 tile (at most 4); the loads are unconditional (clamped), a branch per load costs more.
+    float biasEarly[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) biasEarly[q] = bias[min(o0 + min((tid + q * (64 * KW)) >> 4, 15), O - 1)];
+    }
     for (int j = 0; j < chunks;) {
         load_chunk(aB, bB, j + 1);
         multiply(aA, bA, j);
