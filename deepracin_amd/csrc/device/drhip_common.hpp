@@ -78,6 +78,14 @@ inline FastDiv make_fastdiv(int d) {                 // d >= 1
 }
 __device__ inline int fast_div(int n, const FastDiv& f) { return (int)((__umulhi((unsigned)n, f.mul) + (unsigned)n) >> f.shift); }
 
+// A layer's results are stored written through (system-scope store: sc0 sc1) instead of being left dirty in the
+// XCD's L2: the reader is the next kernel, whose workgroups mostly sit on other XCDs and read from memory anyway,
+// and what has been written during the kernel need not be written back when it ends (0.15-0.45 us per launch on
+// the 14x14 layers, 1.5 us on a 12.8 MB output).
+__device__ inline void store_through(float* p, float v) {
+    __hip_atomic_store((unsigned*)p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // Element `row` of an activation vector that a split GEMV left as partial sums: slices added in
 // order, then bias and ReLU -- bit for bit what the GEMV's finishing kernel stores.
 __device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {

@@ -99,7 +99,7 @@ conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, c
             if (o < O && pOk) {
                 float v = acc[r] + (bias ? bias[o] : 0.0f);
                 if (relu) v = fmaxf(v, 0.0f);
-                out[(size_t)o * P + p0 + l32] = v;
+                store_through(out + (size_t)o * P + p0 + l32, v);
             }
         }
         return;
@@ -125,9 +125,9 @@ conv1x1_mfma_kernel(const float* __restrict__ in, const float* __restrict__ w, c
             s = p < P ? s : 0.0f;
 #pragma unroll
             for (int m = 16; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
-            if (pl == 0 && o < O) poolPartials[(size_t)(p0 >> 5) * O + o] = s;
+            if (pl == 0 && o < O) store_through(poolPartials + (size_t)(p0 >> 5) * O + o, s);
         } else if (o < O && p < P) {
-            out[(size_t)o * P + p] = s;
+            store_through(out + (size_t)o * P + p, s);
         }
     }
 }
@@ -260,7 +260,7 @@ conv1x1_mfma16_kernel(const float* __restrict__ in, const float* __restrict__ w,
         if (o < O && p < P) {
             s += biasEarly[q];
             if (relu) s = fmaxf(s, 0.0f);
-            out[(size_t)o * P + p] = s;
+            store_through(out + (size_t)o * P + p, s);
         }
     }
 }

@@ -279,7 +279,7 @@ conv3x3_fewc_pool3s2_kernel(const float* __restrict__ in, const float* __restric
                     const float v = convT[ch * kFpPitch + (2 * ppy + dy) * kFpConv + 2 * ppx + dx];
                     if (v > r) r = v;
                 }
-            out[((size_t)(o0 + ch) * Hp + py) * Wp + px] = r;
+            store_through(out + ((size_t)(o0 + ch) * Hp + py) * Wp + px, r);
         }
     }
 }
@@ -356,7 +356,7 @@ conv3x3_fewc_mfma_kernel(const float* __restrict__ in, const float* __restrict__
                 if (o0 + ch < O) {
                     float v = acc[m][r] + biasT[ch];
                     if (relu) v = fmaxf(v, 0.0f);
-                    out[((size_t)(o0 + ch) * Ho + y) * Wo + x] = v;
+                    store_through(out + ((size_t)(o0 + ch) * Ho + y) * Wo + x, v);
                 }
             }
     }
@@ -558,7 +558,7 @@ conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict
         if (o < O && pp < P) {
             v += biasValue;
             if (relu) v = fmaxf(v, 0.0f);
-            out[(size_t)o * P + pp] = v;
+            store_through(out + (size_t)o * P + pp, v);
         }
     };
 #pragma unroll

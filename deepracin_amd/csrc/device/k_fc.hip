@@ -146,9 +146,9 @@ fc_gemv_kernel(const float* __restrict__ Wt, const float* __restrict__ x, int K,
         if (slices == 1) {
             if (bias) s += bias[n];
             if (relu) s = fmaxf(s, 0.0f);
-            y[n] = s;
+            store_through(y + n, s);
         } else {
-            partials[(size_t)slice * N + n] = s;
+            store_through(partials + (size_t)slice * N + n, s);
         }
     }
 }
@@ -172,7 +172,7 @@ fc_reduce_kernel(const float* __restrict__ partials, const float* __restrict__ b
     for (; sl < slices; ++sl) s += pp[(size_t)sl * N];
     if (bias) s += bias[n];
     if (relu) s = fmaxf(s, 0.0f);
-    y[n] = s;
+    store_through(y + n, s);
 }
 
 __global__ void __launch_bounds__(256)

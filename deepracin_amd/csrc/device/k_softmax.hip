@@ -72,7 +72,7 @@ softmax_kernel(const float* x, float* y, int n, drhip_deferred_vec xdef) {     /
 #pragma unroll
         for (int u = 0; u < kSoftmaxRegs; ++u) {
             const int i = tid + u * kSoftmaxThreads;
-            if (i < n) y[i] = v[u] * inv;
+            if (i < n) store_through(y + i, v[u] * inv);
         }
         return;
     }
@@ -90,7 +90,7 @@ softmax_kernel(const float* x, float* y, int n, drhip_deferred_vec xdef) {     /
     float s = 0.0f;
     for (int i = tid; i < n; i += kSoftmaxThreads) s += expf(x[i] - m);
     const float inv = 1.0f / block_reduce<false>(s, red);
-    for (int i = tid; i < n; i += kSoftmaxThreads) y[i] = expf(x[i] - m) * inv;
+    for (int i = tid; i < n; i += kSoftmaxThreads) store_through(y + i, expf(x[i] - m) * inv);
 }
 
 }  // namespace drhip
