@@ -129,7 +129,8 @@ int drhip_conv2d_direct_f32(const float* in, const float* w, const float* bias, 
  * order) | 0x10 for 64 instead of 32 output channels per workgroup.  Same function as
  * drhip_conv2d_direct_f32 with kw = kh = 3.  Replaces the per-layer generated kernel
  * `conv2d3x3x<O>_<id>_...` and its launch (src/dR_nodes_conv2d.c:364-420, 481-773); the reference
- * re-lays nothing (it reads [I][O][3][3] through __constant or global memory). */
+ * re-lays nothing (it reads [I][O][3][3] through __constant or global memory).
+ * W, H, I and O at most 65535 each (packed kernel arguments). */
 size_t drhip_conv3x3_direct_filter_floats(int I, int O);
 int drhip_conv3x3_direct_filter_layout_f32(const float* w /* [I][O][3][3] */, float* F, int I, int O, void* stream);
 int drhip_conv3x3_direct_pick_variant(int Wo, int Ho, int I, int O);
@@ -139,7 +140,8 @@ int drhip_conv3x3_direct_mfma_f32(const float* in, const float* F, const float* 
 /* First layer (1 to 4 input channels, 3x3, any stride, zero padding, bias, optional ReLU) followed by
  * a 3x3 / stride-2 max pooling with the reference's pooling rules (out = ceil(in/2), samples outside
  * the map read 0.0): out[O][ceil(Ho/2)][ceil(Wo/2)], Wo = W/strideX, Ho = H/strideY.  The
- * convolution's own tensor is never written.  Replaces the generated conv kernel plus the generated
+ * convolution's own tensor is never written.  W, H and O at most 65535, strides at most 15 (packed kernel
+ * arguments).  Replaces the generated conv kernel plus the generated
  * pooling kernel of such a pair (src/dR_nodes_conv2d.c:481-773, src/dR_nodes_pooling.c:277-401). */
 int drhip_conv3x3_pool3s2_f32(const float* in, const float* w, const float* bias, float* out,
                               int W, int H, int I, int O, int strideX, int strideY, int relu, void* stream);
@@ -160,7 +162,9 @@ int drhip_winograd_filter_transform_f32(const float* w /* [I][O][3][3] */, float
  * workgroup (1: 32, 2: 64, 3: 128), bits 4-7 = log2 of the number of input-channel splits, 0x100 =
  * blocks of 16 tiles (channels per workgroup then 16, 32, 64), 0x400 = eight waves per workgroup (two
  * wave sets that take alternate 8-channel stages; not with 32-tile blocks of 128 channels); 0 lets
- * the launcher pick.  The input must be smaller than 2 GiB (32-bit byte offsets).  A variant that splits the
+ * the launcher pick.  The input must be smaller than 2 GiB (32-bit byte offsets) and W, H, I and O at most 65535
+ * each (the kernel carries them in 16-bit fields of its packed arguments; the graph layer sends larger layers to
+ * drhip_conv2d_direct_f32).  A variant that splits the
  * input channels needs `workspace` of drhip_conv3x3_winograd_workspace_floats(...) floats (scratch,
  * no initialisation needed; two launches: partial tiles, then their sum in split order); otherwise
  * workspace may be NULL.  `relu` is a set of epilogue flags: DRHIP_EPILOGUE_RELU (1) and
