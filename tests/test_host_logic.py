@@ -479,6 +479,34 @@ def test_matmul_helpers():
     assert raw.dR_matmul(a.ctypes.data_as(fp), 4, 3, bt.ctypes.data_as(fp), 6, 3, out2.ctypes.data_as(fp)) == 0
 
 
+def _kernel_line(node):
+    """The 'Kernel: ...' line of a conv node's printLayer text (which algorithm schedule() settled on)."""
+    fn = ctypes.CFUNCTYPE(ctypes.c_void_p, ctypes.c_void_p)(dr.node_struct(node).printLayer)
+    text = ctypes.string_at(fn(node.ptr)).decode()
+    return [l for l in text.splitlines() if "Kernel:" in l][0]
+
+
+def test_layers_beyond_the_packed_argument_fields_take_the_general_kernel(lib):
+    """The matrix-core convolution kernels carry W, H, I and O in 16-bit fields: a 3x3 layer with a dimension above
+    65535 is scheduled onto the general direct kernel, and a first layer of that size is not fused with its pool."""
+    rng = np.random.default_rng(0)
+    for width, expect in ((64, "Winograd"), (70000, "direct")):
+        with dr.Environment() as env:
+            g = env.create_graph()
+            x = dr.feed_node(g, [2, width, 1])                                   # HWC: 2 rows, `width` columns
+            c = dr.Conv2d_raw(x, rng.standard_normal((1, 2, 3, 3)), None, (1, 1), "relu")
+            p = dr.Pooling(c, "max", [1, 3, 3, 1], [1, 2, 2, 1])
+            dr.mark_as_output(p)
+            assert lib.dR_propagateShapesAndSchedule(g.ptr) == 1
+            assert expect in _kernel_line(c), _kernel_line(c)
+            assert lib.dR_planBuffers(g.ptr) == 1
+            # (the conv is a "first layer": with the stride-1 3x3 filter it is a Winograd node, never the fused
+            # first-layer + pool kernel; the wide one, now direct, must not be fused either)
+            plan = plan_of(g, [c, p])
+            if width > 65535:
+                assert plan[0][0] != plan[1][0]                  # the convolution keeps a tensor of its own
+
+
 def test_pick_variants_are_launchable(lib):
     for (W, H, I, O) in [(224, 224, 3, 64), (224, 224, 64, 64), (56, 56, 256, 256), (14, 14, 512, 512), (55, 55, 16, 64), (1, 1, 1, 1)]:
         v = lib.drhip_conv3x3_winograd_pick_variant(W, H, I, O)
