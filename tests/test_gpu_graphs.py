@@ -313,6 +313,28 @@ def test_normalization_behind_an_odd_volume_producer_in_a_concat(oracle, gpu):
         assert_close(got, want[3], "concat %s" % ins)
 
 
+def test_layer_wider_than_the_packed_argument_fields(oracle, gpu):
+    """A 3x3 layer on a 70000 x 2 map (a width beyond the 16-bit fields the matrix-core kernels carry their shapes
+    in) runs on the general direct kernel and gives the oracle's values, with a pooling behind it unfused."""
+    rng = np.random.default_rng(6)
+    W, H = 70000, 2
+    w = (rng.standard_normal((1, 2, 3, 3)) * 0.3).astype(np.float32)
+    b = (rng.standard_normal(2) * 0.1).astype(np.float32)
+    x = rng.standard_normal((1, H, W)).astype(np.float32)
+    spec = [{"op": "feed", "shape": (W, H, 1)},
+            {"op": "conv", "in": 0, "w": w, "b": b, "stride": (1, 1), "relu": True},
+            {"op": "pool", "in": 1, "window": (3, 3, 1), "stride": (2, 2, 1), "kind": 0}]
+    want = oracle.run_spec(spec, {0: x})
+    with dr.Environment() as env:
+        g = env.create_graph()
+        nodes = configs.build_graph(g, spec, [2])
+        dr.prepare(g)
+        configs.feed_chw(nodes[0], x)
+        assert g.lib.dR_apply(g.ptr)
+        got = configs.fetch_chw(g)[0]
+    assert_close(got, want[2], "pool behind a 70000-wide 3x3 layer", terms=9)
+
+
 def test_config4_squeezenet(oracle, gpu):
     spec, feeds, got = run_config("squeezenet", outputs=all_compute_nodes)
     want = check_layers(oracle, spec, feeds, got)
