@@ -257,12 +257,12 @@ int drhip_fc_ex_f32(const float* x, const drhip_deferred_vec* xdef, const float*
                     float* partials, int K, int N, int relu, int defer, void* stream);
 /* drhip_fc_f32 for callers that cannot allocate device memory and have none to lend (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
- * reference.  Same result, bit for bit, as drhip_fc_f32; the partial sums live in a 1 MiB array that
+ * reference.  Same result, bit for bit, as drhip_fc_f32; the partial sums live in a 256 KiB array that
  * is part of the library's code object (one copy per GPU, held until the process ends, its address
  * looked up by drhip_init, which must have run for the current device).  The call allocates and
  * frees nothing.  Shapes whose partial sums exceed drhip_fc_noalloc_max_scratch_floats() floats
  * (drhip_fc_scratch_floats(K,N) tells) are refused with DRHIP_EINVAL; VGG16's three layers need
- * 229376, 65536 and 16000.  All calls on one GPU share the array: calls that may overlap (different
+ * 65536, 65536 and 16000 (the limit is 65536; matrices of 33 000 to 65 000 columns need up to twice that).  All calls on one GPU share the array: calls that may overlap (different
  * streams, or graph branches) race on it; calls on one stream are safe.  Refused while
  * drhip_timing_begin is active. */
 size_t drhip_fc_noalloc_max_scratch_floats(void);
