@@ -33,8 +33,12 @@ __global__ void copy_f32_kernel(float* __restrict__ dst, const float* __restrict
 }
 
 // One workgroup copies n floats into host memory and then raises a flag there, so that the host can watch for
-// the flag instead of waiting for the stream (each lane releases its own stores to system scope, the
-// workgroup meets, lane 0 stores the flag).
+// the flag instead of waiting for the stream.  Release of the data, spelled out: every lane stores with system
+// scope (written through all caches, nothing of it stays dirty in L2, which is all the cache write-back of a
+// system-scope release fence would add), waits until its stores have completed (vmcnt(0): what such a fence waits
+// for as well), the workgroup meets, and only then lane 0 stores the flag, again with system scope.  The host
+// reads the flag with an acquire load before it touches the data.  (The fence itself, __threadfence_system() in
+// every lane, made the download slower than waiting for the stream: 35 against 29 us.)
 __global__ void __launch_bounds__(1024) copy_then_flag_kernel(float* __restrict__ dst, const float* __restrict__ src, size_t n,
                                                               unsigned* flag, unsigned value) {
     for (size_t i = threadIdx.x; i < n; i += blockDim.x)
