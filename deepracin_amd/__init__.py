@@ -171,6 +171,8 @@ def load_library(path=None):
         "drhip_conv3x3_winograd_filter_floats": (c_size_t, [c_int, c_int]),
         "drhip_conv3x3_winograd_workspace_floats": (c_size_t, [c_int] * 5),
         "drhip_conv3x3_winograd_pick_variant": (c_int, [c_int] * 4),
+        "drhip_conv3x3_winograd_workspace_prepare_f32": (c_int, [vp, c_size_t, vp]),
+        "drhip_conv3x3_winograd_join_timeouts": (c_int, [POINTER(ctypes.c_uint)]),
         "drhip_conv1x1_f32": (c_int, [vp, vp, vp, vp] + [c_int] * 5 + [vp]),
         "drhip_conv1x1_pick_variant": (c_int, [c_int] * 3),
         "drhip_conv3x3_direct_filter_floats": (c_size_t, [c_int, c_int]),

@@ -20,10 +20,13 @@
 // Workgroup ids are remapped so that each XCD (own L2) works on a contiguous range of
 // output-channel panels and therefore touches only its share of U.
 // Layers with few tiles cannot fill 256 CUs with panels alone: there the input channels are split
-// over gridDim.y workgroups whose partial outputs are summed, in fixed order, by a small second
-// kernel (deterministic, no float atomics, no device-scope fences).
+// over several workgroups whose partial outputs are summed in fixed order (deterministic, no float
+// atomics, no device-scope fences) - by a small second kernel, or, when all workgroups of the launch
+// are resident at once, by the splits themselves: every split finishes a slice of its panel and
+// waits for the other splits' partial tiles by watching the workspace slots themselves.
 #include "drhip_common.hpp"
 
+#include <cstdlib>
 #include <type_traits>
 
 namespace drhip {
@@ -150,20 +153,31 @@ __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, 
 // is a round trip of its own at the start of every workgroup (~0.07 us each).
 //   wh = W | H << 16, io = I | O << 16 (each at most 65535),
 //   mulX, mulTB = multipliers of the divisions by tilesX and by the number of tile panels,
-//   cfg0 = shiftX | shiftTB << 5 | epilogue flags << 10 (2 bits) | vec2 << 12 | splits << 13,  cfg1 = chunks per split
+//   cfg0 = shiftX | shiftTB << 5 | epilogue flags << 10 (2 bits) | vec2 << 12 | splits << 13 (16 bits) | joined << 31,
+//   cfg1 = chunks per split (16 bits) | log2 splits << 24 (joined launches)
 #define WINO_ARGS unsigned wh, unsigned io, unsigned mulX, unsigned mulTB, unsigned cfg0, unsigned cfg1
 #define WINO_UNPACK(TBV, OBV)                                                                           \
     const int W = (int)(wh & 0xffffu), H = (int)(wh >> 16), I = (int)(io & 0xffffu), O = (int)(io >> 16); \
     const int tilesX = (W + 1) >> 1, T = tilesX * ((H + 1) >> 1);                                         \
     const int nTB = (T + (TBV) - 1) / (TBV), nBlocks = nTB * ((O + (OBV) - 1) / (OBV));                   \
     const FastDiv tilesXd = {(unsigned)tilesX, mulX, cfg0 & 31u}, nTBd = {(unsigned)nTB, mulTB, (cfg0 >> 5) & 31u}; \
-    const int relu = (int)((cfg0 >> 10) & 3u), vec2 = (int)((cfg0 >> 12) & 1u), nSplits = (int)(cfg0 >> 13); \
-    const int chunksPerSplit = (int)cfg1;
+    const int relu = (int)((cfg0 >> 10) & 3u), vec2 = (int)((cfg0 >> 12) & 1u), nSplits = (int)((cfg0 >> 13) & 0xffffu); \
+    const bool joined = (cfg0 >> 31) != 0u;                                                              \
+    const int chunksPerSplit = (int)(cfg1 & 0xffffu), lgSplits = (int)((cfg1 >> 24) & 15u);
 struct WinoPackedArgs { unsigned wh, io, mulX, mulTB, cfg0, cfg1; };
 
 constexpr unsigned kBufferFlags = 0x00020000u;      // dword 3 of a gfx9 raw buffer resource (32-bit data format)
 constexpr int kEpiRelu = DRHIP_EPILOGUE_RELU, kEpiMaxPool2 = DRHIP_EPILOGUE_MAXPOOL2;   // bits of the `relu` argument
 constexpr unsigned kOutOfRange = 0x80000000u;       // byte offset no resource of at most 2 GiB contains
+
+// Joined splits (see the kernel's epilogue).
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+constexpr unsigned kWinoEmpty = 0xffa5c3e1u;        // a signalling NaN: marks a workspace slot whose partial tile has not arrived
+constexpr int kWinoMaxJoin = 8;                     // most splits a joined launch can have
+constexpr int kWinoJoinSpins = 1 << 18;             // bound on the wait for a partner's partial tile (some 0.2 s)
+constexpr int kAuxThrough = 1 | 16;                 // cache policy of a buffer access: sc0 sc1, written through to memory
+constexpr int kAuxDeviceVolatile = 16 | (int)0x80000000u;   // sc1 (device scope: not served from this CU's vector cache), reloaded every time
+__device__ unsigned g_wino_join_timeouts;           // partial tiles that never arrived, over the life of the process
 
 __device__ inline f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset, unsigned soffset) {
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (int)voffset, (int)soffset, 0));
@@ -184,12 +198,15 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
 
     // ---- which panel: XCD-aware remap of the linear workgroup id -----------------------------
     const int perXcd = (nBlocks + kXcds - 1) / kXcds;   // the grid is padded to a multiple of kXcds
-    const int logical = (blockIdx.x % kXcds) * perXcd + blockIdx.x / kXcds;
-    if (logical >= nBlocks) return;
+    // Joined launch: one grid row; the splits of a panel are the workgroups j = id / 8 of one XCD with equal
+    // j >> lgSplits, so they share that XCD's L2 and are dispatched within 8 * splits workgroups of each other.
+    const int slot = joined ? (int)(blockIdx.x / kXcds) >> lgSplits : (int)(blockIdx.x / kXcds);
+    const int logical = (blockIdx.x % kXcds) * perXcd + slot;
+    if (slot >= perXcd || logical >= nBlocks) return;
     const int oBlock = fast_div(logical, nTBd);
     const int o0 = oBlock * OB;
     const int t0 = (logical - oBlock * (int)nTBd.d) * TB;
-    const int split = blockIdx.y;
+    const int split = joined ? (int)(blockIdx.x / kXcds) & (nSplits - 1) : (int)blockIdx.y;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int waveId = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -256,7 +273,7 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     constexpr bool kBiasEarly = NT <= 2;
     constexpr int EO = 8 * KW;                      // output channels finished per pass of the epilogue
     float biasEarly[kBiasEarly ? OB / EO : 1];
-    if (kBiasEarly && bias && nSplits == 1) {
+    if (kBiasEarly && bias && (nSplits == 1 || joined)) {
 #pragma unroll
         for (int q = 0; q < OB / EO; ++q) biasEarly[q] = bias[min(o0 + (tid >> 5) + EO * q, O - 1)];
     }
@@ -358,9 +375,8 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     const int eTy = eTileOk ? fast_div(etg, tilesXd) : 0;
     const int ox = eTileOk ? 2 * (etg - eTy * tilesX) : 0, oy = 2 * eTy;
     f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
-#pragma unroll
-    for (int q = 0; q < OB / EO; ++q) {
-        const int ol = eo + EO * q, o = o0 + ol;
+    // this lane's 2x2 tile of channel ol, summed over the rows of the transform (and the wave sets)
+    auto tile_of = [&](int ol) {
         float p[4][2];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -371,8 +387,70 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
                 p[r][1] += P[(((4 + r) * 2 + 1) * OB + ol) * TB + et];
             }
         }
-        float y00 = p[0][0] + p[1][0] + p[2][0], y01 = p[0][1] + p[1][1] + p[2][1];
-        float y10 = p[1][0] - p[2][0] + p[3][0], y11 = p[1][1] - p[2][1] + p[3][1];
+        return f32x4{p[0][0] + p[1][0] + p[2][0], p[0][1] + p[1][1] + p[2][1],
+                     p[1][0] - p[2][0] + p[3][0], p[1][1] - p[2][1] + p[3][1]};
+    };
+    if (joined) {
+        // Every split finishes the channels ol with ol >> lgRows == split of its panel (OB >> lgSplits channels).
+        // First the partial tiles the other splits are waiting for go out, written through; then this split
+        // collects theirs.  A workspace slot holds kWinoEmpty (a signalling NaN, which no addition can produce)
+        // until its partial tile has been stored, so a reader sees from the slot itself whether the data has
+        // arrived: no flag, no counter, no wait for the stores to complete.  The reader puts kWinoEmpty back.
+        const int lgRows = __builtin_ctz(OB) - lgSplits;
+        const __amdgpu_buffer_rsrc_t rWs = __builtin_amdgcn_make_buffer_rsrc((void*)ws, 0, 0x7ffffff0, kBufferFlags);
+        const unsigned panelFloats = (unsigned)(OB * TB * 4);
+        auto slot_of = [&](int sp, int ol) { return 4u * (((unsigned)sp * (unsigned)nBlocks + (unsigned)logical) * panelFloats + (unsigned)(ol * TB + et) * 4u); };
+#pragma unroll
+        for (int q = 0; q < OB / EO; ++q) {
+            const int ol = eo + EO * q;
+            if ((ol >> lgRows) == split) continue;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, tile_of(ol)), rWs, (int)slot_of(split, ol), 0, kAuxThrough);
+        }
+        const u32x4 empty = {kWinoEmpty, kWinoEmpty, kWinoEmpty, kWinoEmpty};
+#pragma unroll
+        for (int q = 0; q < OB / EO; ++q) {
+            const int ol = eo + EO * q, o = o0 + ol;
+            if ((ol >> lgRows) != split) continue;
+            const f32x4 own = tile_of(ol);
+            u32x4 part[kWinoMaxJoin];
+            bool ready = false;
+            for (int spins = 0; spins < kWinoJoinSpins && !ready; ++spins) {
+                ready = true;
+#pragma unroll
+                for (int u = 0; u < kWinoMaxJoin; ++u)
+                    if (u < nSplits && u != split) part[u] = __builtin_amdgcn_raw_buffer_load_b128(rWs, (int)slot_of(u, ol), 0, kAuxDeviceVolatile);
+#pragma unroll
+                for (int u = 0; u < kWinoMaxJoin; ++u)
+                    if (u < nSplits && u != split)
+                        ready = ready && part[u][0] != kWinoEmpty && part[u][1] != kWinoEmpty && part[u][2] != kWinoEmpty && part[u][3] != kWinoEmpty;
+            }
+            f32x4 s = {0.f, 0.f, 0.f, 0.f};         // splits added in order, like winograd_split_reduce_kernel
+#pragma unroll
+            for (int u = 0; u < kWinoMaxJoin; ++u)
+                if (u < nSplits) s += (u == split) ? own : __builtin_bit_cast(f32x4, part[u]);
+#pragma unroll
+            for (int u = 0; u < kWinoMaxJoin; ++u)
+                if (u < nSplits && u != split) __builtin_amdgcn_raw_buffer_store_b128(empty, rWs, (int)slot_of(u, ol), 0, kAuxThrough);
+            if (!ready) {                           // a partner never delivered: say so in the result and in the counter
+                s = f32x4{__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
+                atomicAdd(&g_wino_join_timeouts, 1u);
+            }
+            if (eTileOk && o < O) {
+                if (bias) s += kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o];
+                if (relu & kEpiRelu) { s[0] = fmaxf(s[0], 0.f); s[1] = fmaxf(s[1], 0.f); s[2] = fmaxf(s[2], 0.f); s[3] = fmaxf(s[3], 0.f); }
+                if (relu & kEpiMaxPool2)
+                    store1_through(out + (size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+                else
+                    wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, s[0], s[1], s[2], s[3]);
+            }
+        }
+        return;
+    }
+#pragma unroll
+    for (int q = 0; q < OB / EO; ++q) {
+        const int ol = eo + EO * q, o = o0 + ol;
+        const f32x4 y = tile_of(ol);
+        float y00 = y[0], y01 = y[1], y10 = y[2], y11 = y[3];
         if (direct) {
             if (eTileOk && o < O) {
                 if (bias) { const float bv = kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
@@ -409,6 +487,7 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
                            WINO_ARGS, float* __restrict__ out, float* __restrict__ ws) {
     constexpr int TB = 16, OB = 16 * NB, KC = kWinoKC;
     WINO_UNPACK(TB, OB)
+    (void)joined; (void)lgSplits;                   // (joined splits exist for 32-tile blocks only)
     extern __shared__ float P[];                    // epilogue only: [KW sets][4 rows][2][OB o][16 t] floats
 
     const int perXcd = (nBlocks + kXcds - 1) / kXcds;
@@ -604,7 +683,7 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
     const int tilesX = (W + 1) >> 1, T = tilesX * ((H + 1) >> 1);
     const int nTB = (T + TB - 1) >> lgTB, nBlocks = nTB * ((O + OB - 1) >> lgOB);
     const FastDiv tilesXd = {(unsigned)tilesX, mulX, cfg0 & 31u}, nTBd = {(unsigned)nTB, mulTB, (cfg0 >> 5) & 31u};
-    const int relu = (int)((cfg0 >> 10) & 3u), vec2 = (int)((cfg0 >> 12) & 1u), nSplits = (int)(cfg0 >> 13);
+    const int relu = (int)((cfg0 >> 10) & 3u), vec2 = (int)((cfg0 >> 12) & 1u), nSplits = (int)((cfg0 >> 13) & 0xffffu);
     const int perXcd = (nBlocks + kXcds - 1) / kXcds;
     const int j = blockIdx.x / kXcds, jp = j >> lgBpp;
     const int panel = (blockIdx.x % kXcds) * perXcd + jp;
@@ -642,13 +721,18 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
 //         | 0x100: 16-tile blocks (then the low 4 bits mean 1 -> 16, 2 -> 32, 3 -> 64 channels)
 //         | 0x400: eight waves per workgroup, two wave sets sharing the stages (32-tile blocks of 32 or 64 channels,
 //                  or 16-tile blocks)
-struct WinoCfg { int nt, splits, tb, waveSets; };
+//         | 0x800: joined splits - the splits of a panel add their partial tiles up inside the one launch (32-tile
+//                  blocks, 2, 4 or 8 splits, every workgroup of the launch resident at once; the workspace must have
+//                  been through drhip_conv3x3_winograd_workspace_prepare_f32)
+struct WinoCfg { int nt, splits, tb, waveSets; bool joined; };
 
 static bool wino_variant(int variant, WinoCfg* c) {
     c->waveSets = (variant & 0x400) ? 2 : 1;
-    if (variant >> 11) return false;
+    c->joined = (variant & 0x800) != 0;
+    if (variant >> 12) return false;
+    if (c->joined && ((variant & 0x100) || ((variant >> 4) & 0xf) < 1 || ((variant >> 4) & 0xf) > 3)) return false;
     if (c->waveSets == 2 && !(variant & 0x100) && (variant & 0xf) > 2) return false;
-    variant &= ~0x400;
+    variant &= ~0xc00;
     const int lg = (variant >> 4) & 0xf;
     if (lg > 6 || (variant >> 9)) return false;
     c->splits = 1 << lg;
@@ -687,9 +771,13 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
     const size_t ldsBytes = 4 * 2 * OB * TB * sizeof(float);
     const int vec2 = ((W & 1) == 0) && (((size_t)out & 7) == 0);
     const FastDiv dx = make_fastdiv(g.tilesX), dtb = make_fastdiv(g.nTB);
+    const bool joined = c.joined && g.splits > 1;   // (a layer with fewer stages than splits may end up unsplit)
     const WinoPackedArgs pa = {(unsigned)W | (unsigned)H << 16, (unsigned)I | (unsigned)O << 16, dx.mul, dtb.mul,
-                               dx.shift | dtb.shift << 5 | (unsigned)(relu & 3) << 10 | (unsigned)vec2 << 12 | (unsigned)g.splits << 13,
-                               (unsigned)g.chunksPerSplit};
+                               dx.shift | dtb.shift << 5 | (unsigned)(relu & 3) << 10 | (unsigned)vec2 << 12 | (unsigned)g.splits << 13 |
+                                   (joined ? 1u << 31 : 0u),
+                               (unsigned)g.chunksPerSplit | (joined ? (unsigned)__builtin_ctz(g.splits) << 24 : 0u)};
+    // joined: one grid row, the splits of a panel side by side on one XCD (see the kernel)
+    const dim3 grid = joined ? dim3(gridX * g.splits) : dim3(gridX, g.splits);
     if constexpr (TB == 32) {
         if constexpr (NT <= 2) {
             if (c.waveSets == 2) {
@@ -705,20 +793,20 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
                 }
             }
             if (c.waveSets == 2)
-                launch((winograd_f23_mfma_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
+                launch((winograd_f23_mfma_kernel<NT, 2>), grid, dim3(2 * kWinoThreads), 2 * ldsBytes, s,
                        in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
         }
         if (c.waveSets != 2 || NT > 2)
-            launch((winograd_f23_mfma_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
+            launch((winograd_f23_mfma_kernel<NT, 1>), grid, dim3(kWinoThreads), ldsBytes, s,
                    in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
     } else if (c.waveSets == 2)
-        launch((winograd_f23_mfma16_kernel<NT, 2>), dim3(gridX, g.splits), dim3(2 * kWinoThreads), 2 * ldsBytes, s,
+        launch((winograd_f23_mfma16_kernel<NT, 2>), grid, dim3(2 * kWinoThreads), 2 * ldsBytes, s,
                in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
     else
-        launch((winograd_f23_mfma16_kernel<NT, 1>), dim3(gridX, g.splits), dim3(kWinoThreads), ldsBytes, s,
+        launch((winograd_f23_mfma16_kernel<NT, 1>), grid, dim3(kWinoThreads), ldsBytes, s,
                in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
     if (int rc = launched("winograd_f23_mfma_kernel")) return rc;
-    if (g.splits > 1) {
+    if (g.splits > 1 && !joined) {
         launch(winograd_split_reduce_kernel, dim3(gridX * (OB * TB / 256)), dim3(256), 0, s,
                workspace, bias, out, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0,
                pa.cfg1 | (unsigned)__builtin_ctz(TB) << 16 | (unsigned)__builtin_ctz(OB) << 20);
@@ -738,6 +826,13 @@ using namespace drhip;
 //     of 8 channels per split;
 //   - split layers with very long channel loops trade panel width against split count;
 //   - small layers take the 16-tile kernel.
+// 0x800 if a split of 2^lg can be joined: 2 to 8 splits of equal length (a power of two of stages), and the
+// switch DR_WINO_JOIN is not 0.
+static int wino_join_flag(int lg, int nChunks) {
+    static const bool enabled = [] { const char* e = getenv("DR_WINO_JOIN"); return !(e && e[0] == '0'); }();
+    return (enabled && lg >= 1 && lg <= 3 && (nChunks & ((1 << lg) - 1)) == 0) ? 0x800 : 0;
+}
+
 extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     const int T = ((W + 1) / 2) * ((H + 1) / 2);
     const int cus = num_cu();
@@ -756,11 +851,23 @@ extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     // At most one workgroup per CU and at least two stages for each wave set: eight waves per workgroup,
     // so that every SIMD still has two waves to alternate between (56x56 256->256: 23.6 vs 24.8 us;
     // 28x28 512->512 as 112 panels x 2 splits: 26.3 vs 26.9 us for 64-channel panels x 4 splits).
-    if ((panels << lg) <= cus && (nChunks >> lg) >= 4) return 0x400 | code | (lg << 4);
+    // A split whose workgroups are all resident at once (one per CU) adds its partial tiles up inside the launch.
+    if ((panels << lg) <= cus && (nChunks >> lg) >= 4) return 0x400 | code | (lg << 4) | wino_join_flag(lg, nChunks);
     // A split layer that still has 32 or more stages per split: the same number of workgroups as
     // 64-channel panels with twice the splits share each input transform between two MFMA sets.
     if (code == 1 && lg >= 1 && lg < 5 && O >= 64 && (nChunks >> lg) >= 32) return 2 | ((lg + 1) << 4);
     return code | (lg << 4);
+}
+
+extern "C" int drhip_conv3x3_winograd_workspace_prepare_f32(float* workspace, size_t floats, void* stream) {
+    DRHIP_REQUIRE(workspace || floats == 0, "drhip_conv3x3_winograd_workspace_prepare_f32: NULL workspace");
+    if (floats == 0) return DRHIP_OK;
+    return drhip_fill_f32(workspace, __builtin_bit_cast(float, kWinoEmpty), floats, stream);
+}
+
+extern "C" int drhip_conv3x3_winograd_join_timeouts(unsigned* count) {
+    DRHIP_REQUIRE(count, "drhip_conv3x3_winograd_join_timeouts: NULL result pointer");
+    return check(hipMemcpyFromSymbol(count, HIP_SYMBOL(g_wino_join_timeouts), sizeof(unsigned)), "hipMemcpyFromSymbol(join timeouts)");
 }
 
 extern "C" size_t drhip_conv3x3_winograd_filter_floats(int I, int O) {
@@ -797,7 +904,7 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
     DRHIP_REQUIRE((relu & ~(DRHIP_EPILOGUE_RELU | DRHIP_EPILOGUE_MAXPOOL2)) == 0, "drhip_conv3x3_winograd_f32: unknown epilogue flags %d", relu);
     DRHIP_REQUIRE(!(relu & DRHIP_EPILOGUE_MAXPOOL2) || ((W | H) & 1) == 0, "drhip_conv3x3_winograd_f32: the fused 2x2 max pool needs even W and H (got %dx%d)", W, H);
     if (variant == 0) {
-        variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O);
+        variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O) & ~0x800;    // (a joined split needs a prepared workspace: explicit variants only)
         if (!workspace) variant &= 0x50f;          // no workspace offered: stay unsplit
     }
     WinoCfg c;
@@ -805,6 +912,16 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
     const WinoGeom g = wino_geom(W, H, I, O, c);
     DRHIP_REQUIRE(g.splits == 1 || workspace, "drhip_conv3x3_winograd_f32: variant %d splits the input channels and needs a workspace", variant);
     DRHIP_REQUIRE(g.splits <= 65535, "drhip_conv3x3_winograd_f32: too many input-channel splits");
+    if (c.joined && g.splits > 1) {
+        // every workgroup waits for its panel's other splits: all of them have to be resident together
+        const int perCu = c.waveSets == 2 ? 1 : (c.nt == 1 ? 3 : (c.nt == 2 ? 2 : 1));
+        DRHIP_REQUIRE((g.splits & (g.splits - 1)) == 0 && g.splits <= kWinoMaxJoin && g.splits * g.chunksPerSplit == g.nChunks,
+                      "drhip_conv3x3_winograd_f32: variant %#x joins %d splits of %d stages: 2, 4 or 8 equal splits only", variant, g.splits, g.chunksPerSplit);
+        DRHIP_REQUIRE((long long)g.nBlocks * g.splits <= (long long)num_cu() * perCu,
+                      "drhip_conv3x3_winograd_f32: variant %#x needs its %d workgroups resident at once, the device holds %d", variant,
+                      g.nBlocks * g.splits, num_cu() * perCu);
+        DRHIP_REQUIRE((long long)g.splits * g.nBlocks * c.tb * c.nt * c.tb * 16 < (1ll << 31), "drhip_conv3x3_winograd_f32: workspace beyond 2 GiB");
+    }
     hipStream_t s = as_stream(stream);
     if (c.tb == 16) {
         if (c.nt == 1) return launch_wino<1, 16>(in, U, bias, out, workspace, W, H, I, O, relu, c, s);

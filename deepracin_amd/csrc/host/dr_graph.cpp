@@ -344,7 +344,13 @@ gboolean dR_apply(dR_Graph* net) {
 void dR_cleanup(dR_Graph* net, gboolean cleanupcl) {
     const bool talk = verbose(net);
     if (talk) say("Cleaning up deepRACIN...\n");
-    if (net->clConfig->clContext) drhip_stream_sync(net->clConfig->hipStream);
+    if (net->clConfig->clContext) {
+        drhip_stream_sync(net->clConfig->hipStream);
+        unsigned late = 0;      // joined Winograd splits whose partner never delivered (their outputs were set to NaN)
+        if (net->prepared && drhip_conv3x3_winograd_join_timeouts(&late) == DRHIP_OK && late > 0)
+            say("deepRACIN: %u partial tiles of split convolutions never arrived in this process (device shared with other work?); "
+                "the affected outputs were NaN. DR_WINO_JOIN=0 selects the two-kernel form.\n", late);
+    }
     if (net->drGraphExec) { drhip_graph_destroy(net->drGraphExec); net->drGraphExec = NULL; }
     if (net->drStaging) { drhip_staging_destroy(net->drStaging); net->drStaging = NULL; }
     for (int k = 0; k < 4; ++k) { drhip_event_destroy(net->drBranchEvents[k]); net->drBranchEvents[k] = NULL; }

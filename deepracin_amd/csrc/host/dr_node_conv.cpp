@@ -161,6 +161,10 @@ gboolean conv_fill(dR_Graph* net, dR_Node* node) {
         if (ok) ok = !device_failed(net, drhip_stream_sync(stream_of(net)), "winograd filter transform (sync)");
         dR_clMemoryBufferCleanup(net, raw);
         net->clConfig->memConsumptionGPU -= (glong)rawBytes;
+        if (ok && c->workspaceBuf && (c->variant & 0x800))     // joined splits recognise missing partial tiles by a marker
+            ok = !device_failed(net, drhip_conv3x3_winograd_workspace_prepare_f32(
+                                         (float*)c->workspaceBuf, drhip_conv3x3_winograd_workspace_floats(c->ishape.s0, c->ishape.s1, I, O, c->variant),
+                                         stream_of(net)), "winograd workspace");
         if (ok && a && launch_has_bias(c)) {
             std::vector<float> bias((size_t)O, 0.0f);
             if (a->useBias) memcpy(bias.data(), a->biases, (size_t)O1 * sizeof(float));

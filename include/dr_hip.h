@@ -161,8 +161,8 @@ int drhip_winograd_filter_transform_f32(const float* w /* [I][O][3][3] */, float
  * `variant` is the configuration chosen by the scheduler: low 4 bits = output channels per
  * workgroup (1: 32, 2: 64, 3: 128), bits 4-7 = log2 of the number of input-channel splits, 0x100 =
  * blocks of 16 tiles (channels per workgroup then 16, 32, 64), 0x400 = eight waves per workgroup (two
- * wave sets that take alternate 8-channel stages; not with 32-tile blocks of 128 channels); 0 lets
- * the launcher pick.  The input must be smaller than 2 GiB (32-bit byte offsets) and W, H, I and O at most 65535
+ * wave sets that take alternate 8-channel stages; not with 32-tile blocks of 128 channels), 0x800 = joined
+ * splits (below); 0 lets the launcher pick.  The input must be smaller than 2 GiB (32-bit byte offsets) and W, H, I and O at most 65535
  * each (the kernel carries them in 16-bit fields of its packed arguments; the graph layer sends larger layers to
  * drhip_conv2d_direct_f32).  A variant that splits the
  * input channels needs `workspace` of drhip_conv3x3_winograd_workspace_floats(...) floats (scratch,
@@ -182,6 +182,19 @@ int drhip_conv3x3_winograd_f32(const float* in, const float* U, const float* bia
  * work-group search in dR_conv2d_winograd_schedule (src/dR_nodes_conv2d.c:809-1006). */
 int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O);
 size_t drhip_conv3x3_winograd_workspace_floats(int W, int H, int I, int O, int variant);
+/* Variants with bit 0x800 ("joined splits": 32-tile blocks, 2, 4 or 8 equal input-channel splits, all workgroups
+ * of the launch resident at once) add the splits' partial tiles up inside the one launch instead of in a second
+ * kernel: every split finishes a slice of its panel and recognises a partial tile that has not arrived yet by the
+ * marker value its workspace slot still holds.  The workspace of such a variant has to go through
+ * drhip_conv3x3_winograd_workspace_prepare_f32 once (it fills in the marker, a signalling NaN that no sum can
+ * produce); every launch leaves it prepared again, so it must not be shared with anything else and launches that use
+ * it must not overlap.  drhip_conv3x3_winograd_f32 with variant 0 never picks a joined variant.  A partner that does
+ * not deliver within the kernel's bounded wait (about 0.2 s: the device was shared so that the launch was not
+ * resident as a whole) turns the affected outputs into NaN and is counted; drhip_conv3x3_winograd_join_timeouts
+ * reads that count (a synchronous copy).  Environment DR_WINO_JOIN=0 keeps pick_variant from returning such variants.
+ * No counterpart in the reference: its kernel never splits the channel sum (Kernels/dR_winograd2.cl:176-189). */
+int drhip_conv3x3_winograd_workspace_prepare_f32(float* workspace, size_t floats, void* stream);
+int drhip_conv3x3_winograd_join_timeouts(unsigned* count);
 
 /* 1x1 convolution as an fp32 MFMA GEMM out[O][P] = w[O x I] . in[I][P], P = H*W; w is the
  * original [I][O] array (no transpose needed).  Replaces kernel `conv2d1x1`, its launch and the

@@ -169,7 +169,10 @@ def wino_workspace(lib, dev, W, H, I, O, variant):
     n = lib.drhip_conv3x3_winograd_workspace_floats(W, H, I, O, variant)
     if not n:
         return None
-    return dev.put(np.full(n, np.nan, np.float32))        # poison: nothing may be read before it is written
+    ws = dev.put(np.full(n, np.nan, np.float32))          # poison: nothing may be read before it is written
+    if variant & 0x800:                                   # joined splits watch the slots for a marker
+        ok(lib, lib.drhip_conv3x3_winograd_workspace_prepare_f32(ws, n, None))
+    return ws
 
 
 def test_winograd_filter_transform(lib, dev, oracle):
@@ -236,6 +239,61 @@ def test_winograd_fused_maxpool(lib, dev, oracle, variant, W, H, I, O):
     p = dev.empty(64)
     assert lib.drhip_conv3x3_winograd_f32(p, U, None, p, 3, 4, I, O, 2, 1, None, None) == -1      # odd width
     assert lib.drhip_conv3x3_winograd_f32(p, U, None, p, 4, 4, I, O, 4, 1, None, None) == -1      # unknown flag
+
+
+@pytest.mark.parametrize("variant", [0x811, 0x812, 0x821, 0x831, 0xc11, 0xc12, 0xc21, 0xc22, 0xc31])
+@pytest.mark.parametrize("W,H,I,O", [
+    (56, 56, 64, 64), (14, 14, 64, 96), (28, 20, 32, 40), (13, 9, 16, 33), (2, 2, 128, 3), (14, 14, 512, 512),
+])
+def test_winograd_joined_splits(lib, dev, oracle, variant, W, H, I, O):
+    """Variant bit 0x800: the splits of a panel add their partial tiles up inside the one launch.  Same sums in the
+    same order as the two-kernel form, so the results must be bit-identical to it; the workspace must be left
+    holding the marker again; several launches in a row; the pooling epilogue."""
+    chunks = -(-I // 8)
+    per_split = -(-chunks // min(1 << ((variant >> 4) & 0xf), chunks))
+    splits = -(-chunks // per_split)                      # what the launcher makes of the request: no empty split
+    x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
+    U, _ = wino_filters(lib, dev, w)
+    xd, bd = dev.put(x), dev.put(b)
+    out = dev.empty(O * H * W)
+    n = lib.drhip_conv3x3_winograd_workspace_floats(W, H, I, O, variant)
+    nt, two_sets = variant & 0xf, bool(variant & 0x400)
+    groups = -(-(-(-W // 2) * -(-H // 2)) // 32) * -(-O // (32 * nt)) * splits
+    resident = groups <= 256 * (1 if two_sets else {1: 3, 2: 2}[nt])     # MI355X: 256 CUs
+    if splits * per_split != chunks or splits & (splits - 1) or not resident:     # unequal splits, or more workgroups than fit at once: refused
+        assert n > 0
+        assert lib.drhip_conv3x3_winograd_f32(xd, U, bd, out, W, H, I, O, 1, variant, dev.empty(n), None) == -1
+        return
+    ws = wino_workspace(lib, dev, W, H, I, O, variant)
+    plain = variant & ~0x800
+    ws2 = wino_workspace(lib, dev, W, H, I, O, plain)
+    ref = dev.empty(O * H * W)
+    ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, ref, W, H, I, O, 1, plain, ws2, None))
+    want = dev.get(ref, (O, H, W))
+    assert_close(want, oracle.conv_winograd(x, w, b, relu=True), floor=float(np.abs(b).max()))
+    for _ in range(3):
+        ok(lib, lib.drhip_fill_f32(out, 7.0, O * H * W, None))
+        ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, out, W, H, I, O, 1, variant, ws, None))
+        assert np.array_equal(dev.get(out, want.shape), want)
+        assert np.all(dev.get(ws, (n,)).view(np.uint32) == 0xffa5c3e1)
+    if W % 2 == 0 and H % 2 == 0:
+        ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, ref, W, H, I, O, 2, plain, ws2, None))
+        ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, out, W, H, I, O, 2, variant, ws, None))
+        assert np.array_equal(dev.get(out, (O, H // 2, W // 2)), dev.get(ref, (O, H // 2, W // 2)))
+    late = ctypes.c_uint(123)
+    ok(lib, lib.drhip_conv3x3_winograd_join_timeouts(ctypes.byref(late)))
+    assert late.value == 0
+
+
+def test_winograd_joined_refused_when_not_resident(lib, dev):
+    """A joined split needs every workgroup of the launch resident at once; a layer with more panels is refused."""
+    p = dev.empty(64)
+    n = lib.drhip_conv3x3_winograd_workspace_floats(224, 224, 16, 64, 0x811)
+    assert n > 0
+    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 224, 224, 16, 64, 0, 0x811, p, None) == -1
+    assert b"resident" in lib.drhip_last_error()
+    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 8, 8, 16, 16, 0, 0x801, p, None) == -1     # joined, but unsplit
+    assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 8, 8, 16, 16, 0, 0x911, p, None) == -1     # 16-tile blocks
 
 
 def test_winograd_auto_variant_vgg_shapes(lib, dev, oracle):
