@@ -28,6 +28,7 @@
 
 #include <cstdlib>
 #include <type_traits>
+#include <utility>
 
 namespace drhip {
 
@@ -153,8 +154,10 @@ __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, 
 // is a round trip of its own at the start of every workgroup (~0.07 us each).
 //   wh = W | H << 16, io = I | O << 16 (each at most 65535),
 //   mulX, mulTB = multipliers of the divisions by tilesX and by the number of tile panels,
-//   cfg0 = shiftX | shiftTB << 5 | epilogue flags << 10 (2 bits) | vec2 << 12 | splits << 13 (16 bits) | joined << 31,
+//   cfg0 = shiftX | shiftTB << 5 | epilogue flags << 10 (2 bits) | vec2 << 12 | splits << 13 (16 bits) | tiered << 30 | joined << 31,
 //   cfg1 = chunks per split (16 bits) | log2 splits << 24 (joined launches)
+//   tiered launches: the splits field holds log2 splits of up to four tiers (4 bits each) and cfg1 their panel
+//   counts per XCD (8 bits each)
 #define WINO_ARGS unsigned wh, unsigned io, unsigned mulX, unsigned mulTB, unsigned cfg0, unsigned cfg1
 #define WINO_UNPACK(TBV, OBV)                                                                           \
     const int W = (int)(wh & 0xffffu), H = (int)(wh >> 16), I = (int)(io & 0xffffu), O = (int)(io >> 16); \
@@ -162,7 +165,7 @@ __device__ inline void wino_store_tile(float* po, int W, int H, int ox, int oy, 
     const int nTB = (T + (TBV) - 1) / (TBV), nBlocks = nTB * ((O + (OBV) - 1) / (OBV));                   \
     const FastDiv tilesXd = {(unsigned)tilesX, mulX, cfg0 & 31u}, nTBd = {(unsigned)nTB, mulTB, (cfg0 >> 5) & 31u}; \
     const int relu = (int)((cfg0 >> 10) & 3u), vec2 = (int)((cfg0 >> 12) & 1u), nSplits = (int)((cfg0 >> 13) & 0xffffu); \
-    const bool joined = (cfg0 >> 31) != 0u;                                                              \
+    const bool joined = (cfg0 >> 31) != 0u, tiered = ((cfg0 >> 30) & 1u) != 0u;                          \
     const int chunksPerSplit = (int)(cfg1 & 0xffffu), lgSplits = (int)((cfg1 >> 24) & 15u);
 struct WinoPackedArgs { unsigned wh, io, mulX, mulTB, cfg0, cfg1; };
 
@@ -173,7 +176,7 @@ constexpr unsigned kOutOfRange = 0x80000000u;       // byte offset no resource o
 // Joined splits (see the kernel's epilogue).
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 constexpr unsigned kWinoEmpty = 0xffa5c3e1u;        // a signalling NaN: marks a workspace slot whose partial tile has not arrived
-constexpr int kWinoMaxJoin = 8;                     // most splits a joined launch can have
+constexpr int kWinoMaxJoin = 16;                    // most splits a joined launch can have
 constexpr int kWinoJoinSpins = 1 << 18;             // bound on the wait for a partner's partial tile (some 0.2 s)
 constexpr int kAuxThrough = 1 | 16;                 // cache policy of a buffer access: sc0 sc1, written through to memory
 constexpr int kAuxDeviceVolatile = 16 | (int)0x80000000u;   // sc1 (device scope: not served from this CU's vector cache), reloaded every time
@@ -200,13 +203,40 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     const int perXcd = (nBlocks + kXcds - 1) / kXcds;   // the grid is padded to a multiple of kXcds
     // Joined launch: one grid row; the splits of a panel are the workgroups j = id / 8 of one XCD with equal
     // j >> lgSplits, so they share that XCD's L2 and are dispatched within 8 * splits workgroups of each other.
-    const int slot = joined ? (int)(blockIdx.x / kXcds) >> lgSplits : (int)(blockIdx.x / kXcds);
+    // Tiered launch: an XCD's panels come in up to four tiers, each with its own number of splits, in dispatch
+    // order (finest cut first, whole panels last): one workgroup of every full tier lands on each CU, so the
+    // CUs end up with equal numbers of stages although the panel count is no multiple of the CU count.
+    int slot = (int)(blockIdx.x / kXcds), split = (int)blockIdx.y, nSp = nSplits, lgSp = lgSplits, chunksHere = chunksPerSplit;
+    if (tiered) {
+        int jj = slot, base = 0;
+        bool found = false;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int n = (int)((cfg1 >> (8 * k)) & 255u), l = (int)((cfg0 >> (13 + 4 * k)) & 15u);
+            if (!found) {
+                if (jj < (n << l)) { found = true; slot = base + (jj >> l); split = jj & ((1 << l) - 1); lgSp = l; }
+                else { jj -= n << l; base += n; }
+            }
+        }
+        if (!found) return;
+        nSp = 1 << lgSp;
+        chunksHere = ((I + kWinoKC - 1) / kWinoKC) >> lgSp;     // (the launcher makes tiers of equal splits only)
+    } else if (joined) {
+        split = slot & (nSplits - 1);
+        slot >>= lgSplits;
+    }
     const int logical = (blockIdx.x % kXcds) * perXcd + slot;
     if (slot >= perXcd || logical >= nBlocks) return;
     const int oBlock = fast_div(logical, nTBd);
     const int o0 = oBlock * OB;
     const int t0 = (logical - oBlock * (int)nTBd.d) * TB;
-    const int split = joined ? (int)(blockIdx.x / kXcds) & (nSplits - 1) : (int)blockIdx.y;
+    // The fewer stages a workgroup has, the sooner its partial tiles can be on their way: small pieces first,
+    // so that the workgroups that end a CU's work are whole panels, which wait for nobody.
+    if (tiered) {
+        if (lgSp >= 3) __builtin_amdgcn_s_setprio(3);
+        else if (lgSp == 2) __builtin_amdgcn_s_setprio(2);
+        else if (lgSp == 1) __builtin_amdgcn_s_setprio(1);
+    }
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int waveId = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -215,8 +245,8 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     const int l32 = lane & 31, lhi = lane >> 5;
     const int plane = H * W;
     const int nChunksAll = (I + KC - 1) / KC;
-    const int chBegin = split * chunksPerSplit;
-    const int chEnd = min(nChunksAll, chBegin + chunksPerSplit);    // > chBegin: the launcher creates no empty split
+    const int chBegin = split * chunksHere;
+    const int chEnd = min(nChunksAll, chBegin + chunksHere);        // > chBegin: the launcher creates no empty split
     const int Opad = wino_opad(O);
 
     // ---- this lane's tile and the byte offsets of the two window rows it reads ---------------
@@ -273,7 +303,7 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     constexpr bool kBiasEarly = NT <= 2;
     constexpr int EO = 8 * KW;                      // output channels finished per pass of the epilogue
     float biasEarly[kBiasEarly ? OB / EO : 1];
-    if (kBiasEarly && bias && (nSplits == 1 || joined)) {
+    if (kBiasEarly && bias && (nSp == 1 || joined)) {
 #pragma unroll
         for (int q = 0; q < OB / EO; ++q) biasEarly[q] = bias[min(o0 + (tid >> 5) + EO * q, O - 1)];
     }
@@ -368,7 +398,7 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 
     // Left factor A^T over the four rows, bias, ReLU, store: lane -> tile tid%32, channels tid/32 + EO*q.
-    const bool direct = nSplits == 1;
+    const bool direct = nSp == 1;
     const int et = tid & 31, eo = tid >> 5;
     const int etg = t0 + et;
     const bool eTileOk = etg < T;
@@ -390,60 +420,77 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
         return f32x4{p[0][0] + p[1][0] + p[2][0], p[0][1] + p[1][1] + p[2][1],
                      p[1][0] - p[2][0] + p[3][0], p[1][1] - p[2][1] + p[3][1]};
     };
-    if (joined) {
+    if (joined && nSp > 1) {
+        // (the partial tiles go out and are looked for at the highest priority: the other workgroups on this CU
+        // are in their channel loops, and a wave at their priority gets an issue slot only when they stall)
+        if (tiered) __builtin_amdgcn_s_setprio(3);
         // Every split finishes the channels ol with ol >> lgRows == split of its panel (OB >> lgSplits channels).
         // First the partial tiles the other splits are waiting for go out, written through; then this split
         // collects theirs.  A workspace slot holds kWinoEmpty (a signalling NaN, which no addition can produce)
         // until its partial tile has been stored, so a reader sees from the slot itself whether the data has
         // arrived: no flag, no counter, no wait for the stores to complete.  The reader puts kWinoEmpty back.
-        const int lgRows = __builtin_ctz(OB) - lgSplits;
+        const int lgRows = __builtin_ctz(OB) - lgSp;
         const __amdgpu_buffer_rsrc_t rWs = __builtin_amdgcn_make_buffer_rsrc((void*)ws, 0, 0x7ffffff0, kBufferFlags);
         const unsigned panelFloats = (unsigned)(OB * TB * 4);
-        auto slot_of = [&](int sp, int ol) { return 4u * (((unsigned)sp * (unsigned)nBlocks + (unsigned)logical) * panelFloats + (unsigned)(ol * TB + et) * 4u); };
+        // (tiered: a workgroup's partial tiles lie at its own index in the grid, its partners' 8 workgroups apart)
+        const unsigned region0 = tiered ? blockIdx.x - (unsigned)(kXcds * split) : (unsigned)logical;
+        const unsigned regionStep = tiered ? (unsigned)kXcds : (unsigned)nBlocks;
+        // byte address of a slot = region of the split (scalar offset) + place of the tile in the panel (per lane)
+        auto region_of = [&](int sp) { return (int)(4u * (region0 + (unsigned)sp * regionStep) * panelFloats); };
+        auto place_of = [&](int ol) { return (int)(16u * (unsigned)(ol * TB + et)); };
 #pragma unroll
         for (int q = 0; q < OB / EO; ++q) {
             const int ol = eo + EO * q;
             if ((ol >> lgRows) == split) continue;
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, tile_of(ol)), rWs, (int)slot_of(split, ol), 0, kAuxThrough);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, tile_of(ol)), rWs, place_of(ol), region_of(split), kAuxThrough);
         }
         const u32x4 empty = {kWinoEmpty, kWinoEmpty, kWinoEmpty, kWinoEmpty};
+        // (the number of splits as a constant: every access below is unconditional.  The slot of the own split is
+        // read and reset like the others - nobody ever writes it - and its content replaced by the own tile.)
+        auto collect = [&](auto nSplitsConst) {
+            constexpr int S = decltype(nSplitsConst)::value;
 #pragma unroll
-        for (int q = 0; q < OB / EO; ++q) {
-            const int ol = eo + EO * q, o = o0 + ol;
-            if ((ol >> lgRows) != split) continue;
-            const f32x4 own = tile_of(ol);
-            u32x4 part[kWinoMaxJoin];
-            bool ready = false;
-            for (int spins = 0; spins < kWinoJoinSpins && !ready; ++spins) {
-                ready = true;
+            for (int q = 0; q < OB / EO; ++q) {
+                const int ol = eo + EO * q, o = o0 + ol;
+                if ((ol >> lgRows) != split) continue;
+                const f32x4 own = tile_of(ol);
+                u32x4 part[S];
+                bool ready = false;
+                for (int spins = 0; spins < kWinoJoinSpins && !ready; ++spins) {
+                    // (the loads are invariant as far as the compiler can see: without this it issues them once,
+                    // in front of the loop)
+                    asm volatile("" ::: "memory");
+                    ready = true;
 #pragma unroll
-                for (int u = 0; u < kWinoMaxJoin; ++u)
-                    if (u < nSplits && u != split) part[u] = __builtin_amdgcn_raw_buffer_load_b128(rWs, (int)slot_of(u, ol), 0, kAuxDeviceVolatile);
+                    for (int u = 0; u < S; ++u) part[u] = __builtin_amdgcn_raw_buffer_load_b128(rWs, place_of(ol), region_of(u), kAuxDeviceVolatile);
 #pragma unroll
-                for (int u = 0; u < kWinoMaxJoin; ++u)
-                    if (u < nSplits && u != split)
-                        ready = ready && part[u][0] != kWinoEmpty && part[u][1] != kWinoEmpty && part[u][2] != kWinoEmpty && part[u][3] != kWinoEmpty;
+                    for (int u = 0; u < S; ++u)
+                        ready = ready && (u == split || (part[u][0] != kWinoEmpty && part[u][1] != kWinoEmpty && part[u][2] != kWinoEmpty && part[u][3] != kWinoEmpty));
+                }
+                f32x4 s = {0.f, 0.f, 0.f, 0.f};     // splits added in order, like winograd_split_reduce_kernel
+#pragma unroll
+                for (int u = 0; u < S; ++u) s += (u == split) ? own : __builtin_bit_cast(f32x4, part[u]);
+#pragma unroll
+                for (int u = 0; u < S; ++u) __builtin_amdgcn_raw_buffer_store_b128(empty, rWs, place_of(ol), region_of(u), kAuxThrough);
+                if (!ready) {                       // a partner never delivered: say so in the result and in the counter
+                    s = f32x4{__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
+                    atomicAdd(&g_wino_join_timeouts, 1u);
+                }
+                if (eTileOk && o < O) {
+                    if (bias) s += kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o];
+                    if (relu & kEpiRelu) { s[0] = fmaxf(s[0], 0.f); s[1] = fmaxf(s[1], 0.f); s[2] = fmaxf(s[2], 0.f); s[3] = fmaxf(s[3], 0.f); }
+                    if (relu & kEpiMaxPool2)
+                        store1_through(out + (size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+                    else
+                        wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, s[0], s[1], s[2], s[3]);
+                }
             }
-            f32x4 s = {0.f, 0.f, 0.f, 0.f};         // splits added in order, like winograd_split_reduce_kernel
-#pragma unroll
-            for (int u = 0; u < kWinoMaxJoin; ++u)
-                if (u < nSplits) s += (u == split) ? own : __builtin_bit_cast(f32x4, part[u]);
-#pragma unroll
-            for (int u = 0; u < kWinoMaxJoin; ++u)
-                if (u < nSplits && u != split) __builtin_amdgcn_raw_buffer_store_b128(empty, rWs, (int)slot_of(u, ol), 0, kAuxThrough);
-            if (!ready) {                           // a partner never delivered: say so in the result and in the counter
-                s = f32x4{__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
-                atomicAdd(&g_wino_join_timeouts, 1u);
-            }
-            if (eTileOk && o < O) {
-                if (bias) s += kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o];
-                if (relu & kEpiRelu) { s[0] = fmaxf(s[0], 0.f); s[1] = fmaxf(s[1], 0.f); s[2] = fmaxf(s[2], 0.f); s[3] = fmaxf(s[3], 0.f); }
-                if (relu & kEpiMaxPool2)
-                    store1_through(out + (size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
-                else
-                    wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, s[0], s[1], s[2], s[3]);
-            }
-        }
+        };
+        static_assert(kWinoMaxJoin == 16, "the cases below");
+        if (lgSp == 1) collect(std::integral_constant<int, 2>{});
+        else if (lgSp == 2) collect(std::integral_constant<int, 4>{});
+        else if (lgSp == 3) collect(std::integral_constant<int, 8>{});
+        else collect(std::integral_constant<int, 16>{});
         return;
     }
 #pragma unroll
@@ -722,17 +769,23 @@ winograd_split_reduce_kernel(const float* __restrict__ ws, const float* __restri
 //         | 0x400: eight waves per workgroup, two wave sets sharing the stages (32-tile blocks of 32 or 64 channels,
 //                  or 16-tile blocks)
 //         | 0x800: joined splits - the splits of a panel add their partial tiles up inside the one launch (32-tile
-//                  blocks, 2, 4 or 8 splits, every workgroup of the launch resident at once; the workspace must have
+//                  blocks, 2 to 16 splits, every workgroup of the launch resident at once; the workspace must have
 //                  been through drhip_conv3x3_winograd_workspace_prepare_f32)
-struct WinoCfg { int nt, splits, tb, waveSets; bool joined; };
+//         | 0x1000 (with 0x800, split bits 0): tiered joined splits - the panels of an XCD are dealt out in tiers
+//                  of whole panels, halves, quarters, ... so that every CU ends up with about the same number of
+//                  stages (see wino_tiers)
+struct WinoCfg { int nt, splits, tb, waveSets; bool joined, tiered; };
 
 static bool wino_variant(int variant, WinoCfg* c) {
     c->waveSets = (variant & 0x400) ? 2 : 1;
     c->joined = (variant & 0x800) != 0;
-    if (variant >> 12) return false;
-    if (c->joined && ((variant & 0x100) || ((variant >> 4) & 0xf) < 1 || ((variant >> 4) & 0xf) > 3)) return false;
+    c->tiered = (variant & 0x1000) != 0;
+    if (variant >> 13) return false;
+    if (c->tiered && (!c->joined || c->waveSets == 2 || ((variant >> 4) & 0xf) != 0 || (variant & 0xf) > 2)) return false;
+    if (c->joined && !c->tiered && ((variant & 0x100) || ((variant >> 4) & 0xf) < 1 || ((variant >> 4) & 0xf) > 4)) return false;
+    if (c->joined && (variant & 0x100)) return false;
     if (c->waveSets == 2 && !(variant & 0x100) && (variant & 0xf) > 2) return false;
-    variant &= ~0xc00;
+    variant &= ~0x1c00;
     const int lg = (variant >> 4) & 0xf;
     if (lg > 6 || (variant >> 9)) return false;
     c->splits = 1 << lg;
@@ -761,7 +814,39 @@ static WinoGeom wino_geom(int W, int H, int I, int O, const WinoCfg& c) {
     return g;
 }
 
-// Workspace: [splits][panel][o in panel][tile in panel] partial 2x2 tiles (float4 each).
+// Tiers of a balanced launch, per XCD.  An XCD has P panels and `cus` CUs.  Written as P / cus = w + 1/2 + 1/4 + ...
+// (binary digits), the panels fall into a tier of w * cus whole panels, a tier of cus / 2 panels cut into halves,
+// one of cus / 4 panels cut into quarters, and so on: each of these tiers puts one workgroup on every CU (the
+// dispatcher deals the workgroups of a launch out in order, one to each CU before any CU gets a second one), and
+// what is left below the finest cut goes out in that cut.  Pieces are powers of two of stages and never less
+// than one stage; at most four tiers, at most 255 panels in one.  The tiers are launched finest cut first.
+struct WinoTiers { int n[4], lg[4], count, wgsPerXcd, maxLg; };
+
+static bool wino_tiers(int nBlocks, int nChunks, int cus, WinoTiers* t) {
+    *t = WinoTiers{};
+    const int P = ceil_div(nBlocks, kXcds);
+    int maxLg = 0;
+    while (maxLg < 4 && (nChunks & ((2 << maxLg) - 1)) == 0 && (cus >> (maxLg + 1)) >= 1) ++maxLg;
+    auto add = [&](int n, int lg) {
+        if (n <= 0) return true;
+        if (t->count && t->lg[t->count - 1] == lg) { t->n[t->count - 1] += n; return t->n[t->count - 1] <= 255; }
+        if (t->count == 4 || n > 255) return false;
+        t->n[t->count] = n; t->lg[t->count] = lg; ++t->count;
+        return true;
+    };
+    int r = P;
+    if (!add(r / cus * cus, 0)) return false;
+    r %= cus;
+    for (int lg = 1; lg <= maxLg; ++lg)
+        if (r >= (cus >> lg)) { if (!add(cus >> lg, lg)) return false; r -= cus >> lg; }
+    if (!add(r, maxLg)) return false;
+    for (int k = 0; k < t->count / 2; ++k) { std::swap(t->n[k], t->n[t->count - 1 - k]); std::swap(t->lg[k], t->lg[t->count - 1 - k]); }
+    for (int k = 0; k < t->count; ++k) { t->wgsPerXcd += t->n[k] << t->lg[k]; t->maxLg = t->lg[k] > t->maxLg ? t->lg[k] : t->maxLg; }
+    return t->maxLg > 0;
+}
+
+// Workspace: [splits][panel][o in panel][tile in panel] partial 2x2 tiles (float4 each); tiered launches: one
+// panel-sized region per workgroup of the grid.
 template <int NT, int TB>
 static int launch_wino(const float* in, const float* U, const float* bias, float* out, float* workspace,
                        int W, int H, int I, int O, int relu, const WinoCfg& c, hipStream_t s) {
@@ -772,6 +857,17 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
     const int vec2 = ((W & 1) == 0) && (((size_t)out & 7) == 0);
     const FastDiv dx = make_fastdiv(g.tilesX), dtb = make_fastdiv(g.nTB);
     const bool joined = c.joined && g.splits > 1;   // (a layer with fewer stages than splits may end up unsplit)
+    if constexpr (TB == 32) {
+        WinoTiers t;
+        if (c.tiered && wino_tiers(g.nBlocks, g.nChunks, num_cu() / kXcds, &t)) {
+            unsigned lgs = 0, counts = 0;
+            for (int k = 0; k < t.count; ++k) { lgs |= (unsigned)t.lg[k] << (4 * k); counts |= (unsigned)t.n[k] << (8 * k); }
+            launch((winograd_f23_mfma_kernel<NT, 1>), dim3(t.wgsPerXcd * kXcds), dim3(kWinoThreads), ldsBytes, s, in, U, bias,
+                   (unsigned)W | (unsigned)H << 16, (unsigned)I | (unsigned)O << 16, dx.mul, dtb.mul,
+                   dx.shift | dtb.shift << 5 | (unsigned)(relu & 3) << 10 | (unsigned)vec2 << 12 | lgs << 13 | 3u << 30, counts, out, workspace);
+            return launched("winograd_f23_mfma_kernel");
+        }
+    }
     const WinoPackedArgs pa = {(unsigned)W | (unsigned)H << 16, (unsigned)I | (unsigned)O << 16, dx.mul, dtb.mul,
                                dx.shift | dtb.shift << 5 | (unsigned)(relu & 3) << 10 | (unsigned)vec2 << 12 | (unsigned)g.splits << 13 |
                                    (joined ? 1u << 31 : 0u),
@@ -852,7 +948,22 @@ extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     // so that every SIMD still has two waves to alternate between (56x56 256->256: 23.6 vs 24.8 us;
     // 28x28 512->512 as 112 panels x 2 splits: 26.3 vs 26.9 us for 64-channel panels x 4 splits).
     // A split whose workgroups are all resident at once (one per CU) adds its partial tiles up inside the launch.
-    if ((panels << lg) <= cus && (nChunks >> lg) >= 4) return 0x400 | code | (lg << 4) | wino_join_flag(lg, nChunks);
+    // (joined splits of fewer than 16 stages each: four waves, 14x14 512->512 as 8 splits: 10.4 vs 11.1 us)
+    if ((panels << lg) <= cus && (nChunks >> lg) >= 4) {
+        const int join = wino_join_flag(lg, nChunks);
+        return ((join && (nChunks >> lg) < 16) ? 0 : 0x400) | code | (lg << 4) | join;
+    }
+    // Unsplit layers with more 32-channel panels than CUs, but no multiple of them (112x112 128->128: 392 panels,
+    // two on 136 CUs and one on 120): tiers of whole, halved, ... panels even the CUs out (21.1 vs 23.2 us;
+    // 224x224 64->64: 22.7 vs 23.2 us).  With 8 stages and fewer than two whole panels per CU it is a tie.
+    if (lg == 0 && wino_join_flag(1, 2)) {
+        static const bool tiersOn = [] { const char* e = getenv("DR_WINO_TIERS"); return !(e && e[0] == '0'); }();
+        const int cusPerXcd = cus / kXcds, P = ceil_div(ceil_div(T, 32) * ceil_div(O, 32), kXcds);
+        WinoTiers t;
+        if (tiersOn && cusPerXcd > 0 && P >= cusPerXcd && P % cusPerXcd != 0 && (nChunks >= 16 || P >= 2 * cusPerXcd) &&
+            wino_tiers(ceil_div(T, 32) * ceil_div(O, 32), nChunks, cusPerXcd, &t))
+            return 0x1801;
+    }
     // A split layer that still has 32 or more stages per split: the same number of workgroups as
     // 64-channel panels with twice the splits share each input transform between two MFMA sets.
     if (code == 1 && lg >= 1 && lg < 5 && O >= 64 && (nChunks >> lg) >= 32) return 2 | ((lg + 1) << 4);
@@ -879,6 +990,8 @@ extern "C" size_t drhip_conv3x3_winograd_workspace_floats(int W, int H, int I, i
     WinoCfg c;
     if (W <= 0 || H <= 0 || I <= 0 || O <= 0 || !wino_variant(variant, &c)) return 0;
     const WinoGeom g = wino_geom(W, H, I, O, c);
+    WinoTiers t;
+    if (c.tiered) return wino_tiers(g.nBlocks, g.nChunks, num_cu() / kXcds, &t) ? (size_t)t.wgsPerXcd * kXcds * (c.tb * c.nt) * c.tb * 4 : 0;
     if (g.splits <= 1) return 0;
     return (size_t)g.splits * g.nBlocks * (c.tb * c.nt) * c.tb * 4;
 }
@@ -904,7 +1017,9 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
     DRHIP_REQUIRE((relu & ~(DRHIP_EPILOGUE_RELU | DRHIP_EPILOGUE_MAXPOOL2)) == 0, "drhip_conv3x3_winograd_f32: unknown epilogue flags %d", relu);
     DRHIP_REQUIRE(!(relu & DRHIP_EPILOGUE_MAXPOOL2) || ((W | H) & 1) == 0, "drhip_conv3x3_winograd_f32: the fused 2x2 max pool needs even W and H (got %dx%d)", W, H);
     if (variant == 0) {
-        variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O) & ~0x800;    // (a joined split needs a prepared workspace: explicit variants only)
+        variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O);
+        if (variant & 0x1000) variant = (variant & 0xf) == 2 ? 2 : 1;      // (joined splits need a prepared workspace: explicit variants only)
+        variant &= ~0x800;
         if (!workspace) variant &= 0x50f;          // no workspace offered: stay unsplit
     }
     WinoCfg c;
@@ -912,11 +1027,20 @@ extern "C" int drhip_conv3x3_winograd_f32(const float* in, const float* U, const
     const WinoGeom g = wino_geom(W, H, I, O, c);
     DRHIP_REQUIRE(g.splits == 1 || workspace, "drhip_conv3x3_winograd_f32: variant %d splits the input channels and needs a workspace", variant);
     DRHIP_REQUIRE(g.splits <= 65535, "drhip_conv3x3_winograd_f32: too many input-channel splits");
-    if (c.joined && g.splits > 1) {
+    if (c.tiered) {
+        WinoTiers t;
+        if (wino_tiers(g.nBlocks, g.nChunks, num_cu() / kXcds, &t)) {
+            // A workgroup waits for the other splits of its panel, which follow it in dispatch order on the same
+            // XCD: as long as one XCD holds more workgroups than a panel has splits, they all get to run.
+            DRHIP_REQUIRE(workspace, "drhip_conv3x3_winograd_f32: variant %#x joins splits and needs a prepared workspace", variant);
+            DRHIP_REQUIRE((1 << t.maxLg) < num_cu() / kXcds, "drhip_conv3x3_winograd_f32: variant %#x cuts panels into %d pieces, an XCD holds %d workgroups", variant, 1 << t.maxLg, num_cu() / kXcds);
+            DRHIP_REQUIRE((long long)t.wgsPerXcd * kXcds * c.tb * c.nt * c.tb * 16 < (1ll << 31), "drhip_conv3x3_winograd_f32: workspace beyond 2 GiB");
+        }
+    } else if (c.joined && g.splits > 1) {
         // every workgroup waits for its panel's other splits: all of them have to be resident together
         const int perCu = c.waveSets == 2 ? 1 : (c.nt == 1 ? 3 : (c.nt == 2 ? 2 : 1));
         DRHIP_REQUIRE((g.splits & (g.splits - 1)) == 0 && g.splits <= kWinoMaxJoin && g.splits * g.chunksPerSplit == g.nChunks,
-                      "drhip_conv3x3_winograd_f32: variant %#x joins %d splits of %d stages: 2, 4 or 8 equal splits only", variant, g.splits, g.chunksPerSplit);
+                      "drhip_conv3x3_winograd_f32: variant %#x joins %d splits of %d stages: 2, 4, 8 or 16 equal splits only", variant, g.splits, g.chunksPerSplit);
         DRHIP_REQUIRE((long long)g.nBlocks * g.splits <= (long long)num_cu() * perCu,
                       "drhip_conv3x3_winograd_f32: variant %#x needs its %d workgroups resident at once, the device holds %d", variant,
                       g.nBlocks * g.splits, num_cu() * perCu);

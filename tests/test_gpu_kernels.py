@@ -296,8 +296,60 @@ def test_winograd_joined_refused_when_not_resident(lib, dev):
     assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 8, 8, 16, 16, 0, 0x911, p, None) == -1     # 16-tile blocks
 
 
+@pytest.mark.parametrize("variant", [0x1801, 0x1802])
+@pytest.mark.parametrize("W,H,I,O", [
+    (112, 112, 128, 128),    # 49 panels per XCD: one cut into 16, 16 halved, 32 whole
+    (112, 112, 64, 128),     # 8 stages: the finest cut is 8
+    (56, 56, 64, 64), (28, 20, 32, 40), (13, 9, 16, 33), (2, 2, 128, 3), (14, 14, 512, 512),
+    (28, 28, 24, 40),        # 3 stages: nothing to halve, the launch stays unsplit
+    (7, 9, 3, 5),
+])
+def test_winograd_tiered_splits(lib, dev, oracle, variant, W, H, I, O):
+    """Variant bits 0x1800: the panels of an XCD go out in tiers of whole, halved, quartered ... panels whose pieces
+    add their partial tiles up inside the launch.  Against the oracle; repeated launches bit-identical; the
+    workspace left holding the marker; the pooling epilogue equal to the pooled unpooled output."""
+    x, w, b = rnd(I, H, W), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
+    U, _ = wino_filters(lib, dev, w)
+    xd, bd = dev.put(x), dev.put(b)
+    out = dev.empty(O * H * W)
+    n = lib.drhip_conv3x3_winograd_workspace_floats(W, H, I, O, variant)
+    chunks = -(-I // 8)
+    assert (n > 0) == (chunks % 2 == 0)
+    ws = wino_workspace(lib, dev, W, H, I, O, variant)
+    want = oracle.conv_winograd(x, w, b, relu=True)
+    first = None
+    for _ in range(3):
+        ok(lib, lib.drhip_fill_f32(out, 7.0, O * H * W, None))
+        ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, out, W, H, I, O, 1, variant, ws, None))
+        got = dev.get(out, want.shape)
+        assert_close(got, want, floor=float(np.abs(b).max()))
+        first = got if first is None else first
+        assert np.array_equal(got, first)
+        if n:
+            assert np.all(dev.get(ws, (n,)).view(np.uint32) == 0xffa5c3e1)
+    assert_close(first, oracle.conv_f64(x, w, b, relu=True), floor=float(np.abs(b).max()))
+    if W % 2 == 0 and H % 2 == 0:
+        pooled = dev.empty(O * H * W // 4)
+        ok(lib, lib.drhip_conv3x3_winograd_f32(xd, U, bd, pooled, W, H, I, O, 1 | 2, variant, ws, None))
+        assert np.array_equal(dev.get(pooled, (O, H // 2, W // 2)), oracle.pool(first, (2, 2, 1), (2, 2, 1), 0))
+    late = ctypes.c_uint(123)
+    ok(lib, lib.drhip_conv3x3_winograd_join_timeouts(ctypes.byref(late)))
+    assert late.value == 0
+    if n:       # the pieces wait for each other through the workspace: none offered, refused
+        assert lib.drhip_conv3x3_winograd_f32(xd, U, bd, out, W, H, I, O, 1, variant, None, None) == -1
+
+
+def test_winograd_tiered_refused_combinations(lib, dev):
+    p = dev.empty(64)
+    for variant in (0x1001, 0x1901, 0x1c01, 0x1811, 0x1803, 0x2801):     # not joined, 16-tile blocks, two wave sets, split bits, 128 channels, unknown bit
+        assert lib.drhip_conv3x3_winograd_workspace_floats(8, 8, 16, 16, variant) == 0
+        assert lib.drhip_conv3x3_winograd_f32(p, p, None, p, 8, 8, 16, 16, 0, variant, p, None) == -1, hex(variant)
+
+
 def test_winograd_auto_variant_vgg_shapes(lib, dev, oracle):
-    for (W, I, O) in [(56, 128, 256), (28, 256, 512), (14, 512, 512)]:
+    assert lib.drhip_conv3x3_winograd_pick_variant(112, 112, 128, 128) == 0x1801      # (MI355X: 32 CUs per XCD)
+    assert lib.drhip_conv3x3_winograd_pick_variant(14, 14, 512, 512) == 0x831
+    for (W, I, O) in [(224, 64, 64), (112, 128, 128), (56, 128, 256), (28, 256, 512), (14, 512, 512)]:
         x, w, b = np.abs(rnd(I, W, W)), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
         U, _ = wino_filters(lib, dev, w)
         variant = lib.drhip_conv3x3_winograd_pick_variant(W, W, I, O)
