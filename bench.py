@@ -221,7 +221,8 @@ def analyse(lib, m, workload, counters):
             I, O = n["w"].shape[0], joint_o.get(i, n["w"].shape[1])
             issued = winograd_issued_flops(lib, W, H, I, O)
             gk["issued"] += issued
-            if (lib.drhip_conv3x3_winograd_pick_variant(W, H, I, O) >> 4) & 0xf:       # split layers: the partial tiles are summed by a second kernel
+            v = lib.drhip_conv3x3_winograd_pick_variant(W, H, I, O)
+            if (v >> 4) & 0xf and not v & 0x800:       # split layers whose partial tiles are summed by a second kernel
                 gk["kernels"] += 1
             row["issued_tflops"] = round(issued / (ms[i] * 1e-3) / 1e12, 2)
             row["mfma_busy_frac"] = round(issued / (ms[i] * 1e-3) / 1e12 / PEAK_MFMA_F32_TFLOPS, 4)
@@ -252,7 +253,8 @@ def analyse(lib, m, workload, counters):
             # counters of the committed rocprofv3 run: busy cycles per SIMD over THIS run's device time (the profiler's own
             # timestamps run ~10 % long), and the share under the profiler itself
             cyc = rec.get("mfma_busy_cycles_per_simd")
-            roofline.update({"issued_tflops": round(issued, 3), "mfma_busy_frac": round(issued / PEAK_MFMA_F32_TFLOPS, 4),
+            roofline.update({"issued_tflops": round(issued, 3), "frac_issued": round(issued / PEAK_MFMA_F32_TFLOPS, 4),
+                             "mfma_busy_frac": round(issued / PEAK_MFMA_F32_TFLOPS, 4),
                              "mfma_busy_frac_counters": round(cyc / (gk["ms"] * 1e3 * PEAK_CLOCK_GHZ * 1e3), 4) if cyc else None,
                              "mfma_busy_frac_profiled": rec.get("mfma_busy_frac"),
                              "target": "mfma_busy_frac >= 0.50"})
@@ -272,6 +274,27 @@ def analyse(lib, m, workload, counters):
                       "tflops": round(v["flops"] / (v["ms"] * 1e-3) / 1e12, 2) if v["ms"] > 0 and v["flops"] else None}
                   for k, v in groups.items()}
     return layers, out_groups, roofline, roofline_fc
+
+
+def kernel_sources_sha1():
+    """Hash over the device sources (csrc/device): identifies the kernels a profile was taken on."""
+    import hashlib
+    h = hashlib.sha1()
+    d = os.path.join(ROOT, "deepracin_amd", "csrc", "device")
+    for f in sorted(os.listdir(d)):
+        if f.endswith((".hip", ".hpp")):
+            h.update(f.encode())
+            h.update(open(os.path.join(d, f), "rb").read())
+    return h.hexdigest()
+
+
+def compact_roofline(r):
+    """The roofline block without its explanatory strings (for the one-line summary)."""
+    if not r:
+        return r
+    keep = ("kernel", "bound", "achieved", "peak", "unit", "frac", "frac_issued", "traffic", "mfma_busy_frac_counters",
+            "mfma_busy_frac_profiled", "launches_per_step", "avg_launch_ms")
+    return {k: r[k] for k in keep if k in r}
 
 
 def probe_pocl():
@@ -448,6 +471,9 @@ def summarise(dirs, workload, counters_json, last=0):
         print()
     if counters_json and record:
         data = json.load(open(counters_json)) if os.path.exists(counters_json) else {}
+        sha = kernel_sources_sha1()
+        if data.get("kernel_sources_sha1") != sha:      # figures of other kernel sources do not mix with these
+            data = {"kernel_sources_sha1": sha}
         entry = data.setdefault(workload, {})
         for g, rec in record.items():
             rec["measured"] = time.strftime("%Y-%m-%d")
@@ -492,6 +518,10 @@ def main():
         print("bench.py: no HIP device visible; the hot path has no CPU fallback", file=sys.stderr)
         sys.exit(1)
     counters = json.load(open(COUNTERS_JSON)) if os.path.exists(COUNTERS_JSON) else {}
+    # Counter figures belong to the kernels they were measured on: a file written for other kernel sources is not replayed.
+    counters_stale = bool(counters) and counters.get("kernel_sources_sha1") != kernel_sources_sha1()
+    if counters_stale:
+        counters = {}
 
     if args.calibrate_copy:
         calibrate_copy(lib, dr)
@@ -557,6 +587,25 @@ def main():
         for k, gk in groups.items():
             print("%-9s %2d launches %8.4f ms" % (k, gk["launches"], gk["ms"]), file=sys.stderr)
 
+    e2e_ips = round(1e3 / m["e2e_ms"], 1)
+    detail = {
+        "workload": args.workload, "ms_per_step": round(m["ms_per_step"], 4), "timed_blocks": args.blocks,
+        "kernel_ms_per_step": round(float(m["per_node"].sum()), 4),
+        "kernels_per_step": sum(v["kernels"] for v in groups.values()),
+        "roofline": roofline, "roofline_fc": roofline_fc, "groups": groups, "layers": layers,
+        "secondary": secondary, "configs": configs_out, "pocl": pocl, "counters_stale": counters_stale,
+    }
+    # The tables go to stderr (one JSON document); stdout carries ONE short line with both networks of the metric.
+    print("bench.py detail: " + json.dumps(detail), file=sys.stderr)
+    sec_line = None
+    if secondary:
+        sec_line = {k: secondary[k] for k in ("workload", "value", "unit", "ms_per_step", "kernel_ms_per_step", "kernels_per_step")}
+        sec_line["e2e_images_per_s"] = round(1e3 / secondary["e2e_ms_per_step_with_feed_and_download"], 1)
+        sec_line["roofline"] = compact_roofline(secondary["roofline"])
+    cfg_line = None
+    if configs_out:
+        cfg_line = {name: {"ms_per_step": c["ms_per_step"], "kernel_ms": c["gpu_kernels_ms"], "frac": c["frac_of_mfma_peak"],
+                           "mfma_busy_frac": (c["roofline"] or {}).get("mfma_busy_frac")} for name, c in configs_out.items()}
     line = {
         "metric": "batch-1 images/s %s fp32 through dR_apply" % args.workload,
         "value": round(1e3 / m["ms_per_step"], 2),
@@ -567,7 +616,6 @@ def main():
         "ms_per_step": round(m["ms_per_step"], 4),
         "ms_per_step_min": round(m["ms_min"], 4),
         "ms_per_step_max": round(m["ms_max"], 4),
-        "timed_blocks": args.blocks,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -575,18 +623,15 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "batch": 1, "input": list(spec[0]["shape"]), "seed": args.seed,
                    "nodes": len(spec), "conv_gflop": round(sum(v for i, v in flops.items() if spec[i]["op"] == "conv") / 1e9, 3),
-                   "launch_graph": m["launch_graph"]},
-        "roofline": roofline,
-        "roofline_fc": roofline_fc,
+                   "launch_graph": m["launch_graph"], "kernels_per_step": detail["kernels_per_step"],
+                   "kernel_ms_per_step": detail["kernel_ms_per_step"],
+                   "e2e_images_per_s": e2e_ips, "e2e_ms_per_step_with_feed_and_download": round(m["e2e_ms"], 4)},
+        "roofline": compact_roofline(roofline),
+        "roofline_fc": {k: v for k, v in roofline_fc.items() if k != "bytes_per_launch"} if roofline_fc else None,
         "cpu_baseline": cpu_baseline,
-        "pocl": pocl,
-        "secondary": secondary,
-        "configs": configs_out,
-        "kernel_ms_per_step": round(float(m["per_node"].sum()), 4),
-        "kernels_per_step": sum(v["kernels"] for v in groups.values()),
-        "e2e_ms_per_step_with_feed_and_download": round(m["e2e_ms"], 4),
-        "groups": groups,
-        "layers": layers,
+        "secondary": sec_line,
+        "configs": cfg_line,
+        "counters_stale": counters_stale,
     }
     print(json.dumps(line))
 

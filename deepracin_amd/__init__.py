@@ -106,7 +106,8 @@ def load_library(path=None):
         # graph API
         "dR_NewGraph": (vp, []),
         "dR_config": (None, [vp, c_char_p, c_int, c_int, c_int, c_int, c_char_p]),
-        "dR_initCL": (None, [vp]),
+        "dR_initCL": (c_int, [vp]),
+        "dR_getClEnvironmentFrom": (None, [vp, vp]),
         "dR_setAsOutput": (c_int, [vp, vp]),
         "dR_prepare": (c_int, [vp]),
         "dR_getOutputBuffers": (c_int, [vp, POINTER(vp)]),
@@ -257,6 +258,7 @@ class Environment:
     def __init__(self, preferred_platform=""):
         self.preferred_platform_name = preferred_platform
         self.graphs = []
+        self.graph_with_cl_context = -1
         self.id_counter = 0
         self.silent = True
         self.debuginfo = False
@@ -272,11 +274,12 @@ class Environment:
         return False
 
     def close(self):
-        for g in self.graphs:
+        for g in reversed(self.graphs):         # (the first prepared graph owns the stream the later ones borrowed)
             if g.ptr:
                 g.lib.dR_cleanup(g.ptr, 1)
                 g.ptr = None
         self.graphs = []
+        self.graph_with_cl_context = -1
 
     def create_graph(self, interface_layout="HWC"):
         g = Graph(self.id_counter, interface_layout, self)
@@ -313,7 +316,14 @@ def prepare(graph):
     plat, mdir = env.preferred_platform_name.encode(), model_path.encode()
     graph._keep += [plat, mdir]
     graph.lib.dR_config(graph.ptr, plat, int(env.silent), int(env.debuginfo), int(env.profileGPU), int(env.profileCPU), mdir)
-    graph.lib.dR_initCL(graph.ptr)
+    # the first graph of an environment brings the device up, the others take its device and stream (reference :408-428)
+    first = next((g for g in env.graphs if g.id == env.graph_with_cl_context and g.ptr), None)
+    if first is None:
+        if not graph.lib.dR_initCL(graph.ptr):
+            raise RuntimeError("DR Error: deepRACIN initCL failed!")
+        env.graph_with_cl_context = graph.id
+    elif first is not graph:
+        graph.lib.dR_getClEnvironmentFrom(graph.ptr, first.ptr)
     if not graph.lib.dR_prepare(graph.ptr):
         raise RuntimeError("DR Error: deepRACIN prepare failed!")
     for node in graph.outnodes:

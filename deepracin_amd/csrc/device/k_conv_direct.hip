@@ -531,7 +531,9 @@ conv3x3_direct_mfma_kernel(const float* __restrict__ in, const float* __restrict
         }
     };
     // stages whose successor (KW further on) is a complete chunk prefetch in the plain form
-    const int chMain = I / KC - KW;
+    // (plain form only for successor chunks in front of the one with the tensor's last channel: the scalar offset is
+    // not range-checked, and the row loads of the last pixels of the last row reach up to two samples past the row)
+    const int chMain = (I - 1) / KC - KW;
     int ch = wave;
     for (; ch < chMain; ch += KW) stage(ch, std::true_type{});
     for (; ch < nChunks; ch += KW) stage(ch, std::false_type{});

@@ -26,6 +26,7 @@
 // waits for the other splits' partial tiles by watching the workspace slots themselves.
 #include "drhip_common.hpp"
 
+#include <atomic>
 #include <cstdlib>
 #include <type_traits>
 #include <utility>
@@ -370,9 +371,12 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
         load_filters(f[3], 3, next);
         __builtin_amdgcn_sched_barrier(0);
     };
-    // Stages whose successor chunk (KW further on) is complete (all 8 channels exist) prefetch in the
-    // plain form; the last ones of the tensor use the ranged form.
-    const int chMain = min(chEnd, I / KC - KW);
+    // Stages whose successor chunk (KW further on) is complete (all 8 channels exist) and does not hold the
+    // tensor's last channel prefetch in the plain form; the last ones of the tensor use the ranged form.  (The
+    // scalar offset of a buffer access is not part of its range check, and the 16-byte row loads of the last
+    // tiles of the last row reach one or two samples past the row: in the last channel that is past the tensor,
+    // where only the ranged form's resource ends.)
+    const int chMain = min(chEnd, (I - 1) / KC - KW);
     int ch = chBegin + kset;
     for (; ch < chMain; ch += KW) stage(ch, std::true_type{});
     for (; ch < chEnd; ch += KW) stage(ch, std::false_type{});
@@ -656,7 +660,7 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
         load_filters(f[3], 3, next);
         __builtin_amdgcn_sched_barrier(0);
     };
-    const int chMain = min(chEnd, I / KC - KW);
+    const int chMain = min(chEnd, (I - 1) / KC - KW);      // (see the 32-tile kernel)
     int ch = chBegin + kset;
     for (; ch < chMain; ch += KW) stage(ch, std::true_type{});
     for (; ch < chEnd; ch += KW) stage(ch, std::false_type{});
@@ -879,13 +883,15 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
             if (c.waveSets == 2) {
                 // more than 64 KiB of dynamic LDS has to be asked for once per kernel
                 // (the attribute belongs to the kernel's code object on ONE device)
-                static bool raised[64] = {};
+                // (remembered per device; graphs may be prepared and applied from several host threads)
+                static std::atomic<bool> raised[64];
                 int device = 0;
                 if (int rc = check(hipGetDevice(&device), "hipGetDevice")) return rc;
-                if (2 * ldsBytes > 65536 && !(device >= 0 && device < 64 && raised[device])) {
+                const bool known = device >= 0 && device < 64;
+                if (2 * ldsBytes > 65536 && !(known && raised[device].load(std::memory_order_acquire))) {
                     if (int rc = check(hipFuncSetAttribute((const void*)winograd_f23_mfma_kernel<NT, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(2 * ldsBytes)),
                                        "hipFuncSetAttribute(max dynamic LDS)")) return rc;
-                    if (device >= 0 && device < 64) raised[device] = true;
+                    if (known) raised[device].store(true, std::memory_order_release);
                 }
             }
             if (c.waveSets == 2)

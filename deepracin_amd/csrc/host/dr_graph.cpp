@@ -140,7 +140,8 @@ static gboolean ensure_device(dR_Graph* net) {
     return TRUE;
 }
 
-void dR_initCL(dR_Graph* net) { ensure_device(net); }
+// (TRUE on purpose: the reference's Python wrapper reads a bool from this call, see the header)
+gboolean dR_initCL(dR_Graph* net) { return ensure_device(net) ? TRUE : FALSE; }
 
 void dR_setClEnvironment(dR_Graph* net, cl_context, cl_platform_id, cl_command_queue clcommandqueue,
                          cl_device_id) {
@@ -169,8 +170,13 @@ gboolean dR_prepare(dR_Graph* net) {
     // One dR_prepare per graph: the schedule flags of the nodes, the planned buffers and the uploaded
     // weights of the first call are not rolled back, so a second walk would find every node already
     // queued and schedule nothing.  Refused loudly instead of returning a graph that computes nothing.
-    if (net->scheduledLayers || net->prepared) {
+    if (net->prepared) {
         say("dR_prepare: this graph has been prepared already; build a new graph (dR_NewGraph) to prepare again.\n");
+        return FALSE;
+    }
+    if (net->scheduledLayers) {     // scheduled, but never usable: a dR_prepare that failed, or dR_propagateShapesAndSchedule called by hand
+        say("dR_prepare: this graph has been scheduled before (by a dR_prepare that failed, or by a call of "
+            "dR_propagateShapesAndSchedule) and cannot be scheduled a second time; build a new graph (dR_NewGraph).\n");
         return FALSE;
     }
     if (!ensure_device(net)) { say("dR_initCL Failed \n"); return FALSE; }
@@ -251,6 +257,20 @@ void dR_feedData(dR_Graph* net, dR_Node* feednode, gfloat* data, gint offset, gi
 // without waiting; after the last node the pass is awaited once, a node's device time
 // (node->drLastKernelMs) is the sum over its kernels, and their sum goes to
 // clConfig->totalKernelGPUTime, printed like the reference does.
+// Fusions decided by the buffer planner leave some nodes without a stored tensor of their own.
+static bool tensor_fused_away(const dR_Node* n) {
+    if (n->type == tConv2d) {
+        const dR_Conv2d_Data* c = (const dR_Conv2d_Data*)n->layer;
+        return c->drFusedPool || c->drFusedAvgPool;
+    }
+    if (n->type == tPooling && ((const dR_Pooling_Data*)n->layer)->drFused && n->next_layers && n->next_layers->length == 1) {
+        const dR_Node* c = (const dR_Node*)n->next_layers->first->element;
+        return c->type == tConv2d && ((const dR_Conv2d_Data*)c->layer)->drPooledInput == n;
+    }
+    if (n->type == tFullyConnected) return ((const dR_FC_Data*)n->layer)->drDeferReduce && !n->output;
+    return false;
+}
+
 gboolean dR_apply(dR_Graph* net) {
     if (!net->prepared) { say("dR_apply: graph is not prepared. Call dR_prepare first! \n"); return FALSE; }
     dR_ClConfig* cc = net->clConfig;
@@ -308,9 +328,14 @@ gboolean dR_apply(dR_Graph* net) {
             if (profGPU) drhip_timing_end(NULL, 0, NULL);
             return FALSE;
         }
-        if (node->layerID == net->debugLayer && net->hostDebugBuffer)
-            dR_downloadArray(net, (gchar*)"", node->outputBuf->bufptr, 0,
-                             (size_t)node->oshape.s0 * node->oshape.s1 * sizeof(float), net->hostDebugBuffer);
+        if (node->layerID == net->debugLayer && net->hostDebugBuffer) {
+            if (tensor_fused_away(node))
+                say("dR_apply: layer %d is computed inside a neighbouring kernel and its tensor is never stored; set "
+                    "debugLayer before dR_prepare and the buffer planner keeps it.\n", node->layerID);
+            else
+                dR_downloadArray(net, (gchar*)"", node->outputBuf->bufptr, 0,
+                                 (size_t)node->oshape.s0 * node->oshape.s1 * sizeof(float), net->hostDebugBuffer);
+        }
     }
     if (profGPU) {
         firstLaunch.push_back(drhip_timing_count());

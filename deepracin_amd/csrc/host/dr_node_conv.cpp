@@ -75,7 +75,10 @@ gboolean conv_schedule(dR_Graph* net, dR_Node* node) {
     const int W = c->ishape.s0, H = c->ishape.s1, I = c->shape.s2, O = c->shape.s3;
     // The matrix-core convolution kernels carry W, H, I and O in 16-bit fields of their packed arguments;
     // a layer beyond that takes the general direct kernel.
-    const bool packable = W <= 65535 && H <= 65535 && I <= 65535 && O <= 65535;
+    // They also address their input and their filters with 32-bit byte offsets (the entry points refuse 2^29 input
+    // elements or more); such a layer takes the general direct kernel, which indexes with size_t, as well.
+    const bool packable = W <= 65535 && H <= 65535 && I <= 65535 && O <= 65535 && (long long)W * H * I < (1ll << 29) &&
+                          (long long)W * H * O < (1ll << 31) && (long long)(I + 7) * (O + 31) * 16 < (1ll << 29);
     if (c->algo == drConvWinograd && !packable) c->algo = drConvDirect;
     switch (c->algo) {
         case drConvWinograd: c->variant = drhip_conv3x3_winograd_pick_variant(W, H, I, O); break;

@@ -33,6 +33,11 @@ struct Root {
     dR_MemoryHandler* phys = nullptr;
 };
 
+// A node whose tensor has to exist in memory after the pass although the graph has one reader for it: an output
+// node, or the layer the caller asked a debug download of (dR_Graph::debugLayer, read when the buffers are planned).
+thread_local int g_debugLayerAtPlanTime = -1;
+inline bool tensor_wanted(const dR_Node* n) { return n->output || n->layerID == g_debugLayerAtPlanTime; }
+
 bool concat_can_fuse(const dR_Node* c) {
     if (c->type != tConcat) return false;
     const dR_Concat_Data* cd = (const dR_Concat_Data*)c->layer;
@@ -46,7 +51,7 @@ bool concat_can_fuse(const dR_Node* c) {
         // may only sit at a multiple of 4 floats (buffers themselves start 256-byte aligned).
         if (p->type == tNormalization && (off & 3)) return false;
         off += p->oshape.s0 * p->oshape.s1 * p->oshape.s2;
-        if (p->type == tDataFeedNode || p->output) return false;
+        if (p->type == tDataFeedNode || tensor_wanted(p)) return false;
         if (!p->next_layers || p->next_layers->length != 1) return false;
         if (p->outputBuf) return false;     // already bound to a caller buffer
         if (p->oshape.s0 != c->oshape.s0 || p->oshape.s1 != c->oshape.s1) return false;
@@ -91,7 +96,7 @@ dR_Node* pool_fusable_producer(const dR_Node* p) {
     dR_Node* c = ins[0];
     if (c->type != tConv2d) return nullptr;
     const dR_Conv2d_Data* cd = (const dR_Conv2d_Data*)c->layer;
-    if (c->output || c->outputBuf || !c->next_layers || c->next_layers->length != 1) return nullptr;
+    if (tensor_wanted(c) || c->outputBuf || !c->next_layers || c->next_layers->length != 1) return nullptr;
     if (two) {
         if (cd->algo != drConvWinograd || ((c->oshape.s0 | c->oshape.s1) & 1)) return nullptr;
     } else {
@@ -117,8 +122,10 @@ dR_Node* pooled_input_of(const dR_Node* c) {
     const dR_Pooling_Data* pd = (const dR_Pooling_Data*)p->layer;
     if (pd->poolingType != tMax || pd->shape.s1 != 3 || pd->shape.s2 != 3 || pd->shape.s3 != 1) return nullptr;
     if (pd->stride.s1 != 2 || pd->stride.s2 != 2 || pd->stride.s3 != 1) return nullptr;
-    if (p->output || p->outputBuf || !p->next_layers || p->next_layers->length != 1) return nullptr;
+    if (tensor_wanted(p) || p->outputBuf || !p->next_layers || p->next_layers->length != 1) return nullptr;
     if (pool_fusable_producer(p)) return nullptr;      // already stored by the convolution in front of it
+    // (the pooling-on-load kernel addresses the unpooled tensor with 32-bit byte offsets)
+    if ((long long)pd->ishape.s0 * pd->ishape.s1 * pd->ishape.s2 >= (1ll << 29)) return nullptr;
     return p;
 }
 
@@ -141,7 +148,7 @@ dR_Node* avgpool_fusable_producer(const dR_Node* p) {
     if (ins.size() != 1) return nullptr;
     dR_Node* c = ins[0];
     if (c->type != tConv2d || ((const dR_Conv2d_Data*)c->layer)->algo != drConv1x1Gemm) return nullptr;
-    if (c->output || c->outputBuf || !c->next_layers || c->next_layers->length != 1) return nullptr;
+    if (tensor_wanted(c) || c->outputBuf || !c->next_layers || c->next_layers->length != 1) return nullptr;
     return c;
 }
 
@@ -255,6 +262,7 @@ gboolean dR_planBuffers(dR_Graph* net) {
     if (!net->scheduledLayers) { say("dR_planBuffers: graph has no schedule yet\n"); return FALSE; }
     std::vector<dR_Node*> sched = nodes_of(net->scheduledLayers);
     std::vector<dR_Node*> feeds = nodes_of(net->feed_layers);
+    g_debugLayerAtPlanTime = net->debugLayer;
 
     // 1. which concat nodes absorb their producers
     std::map<dR_Node*, std::pair<dR_Node*, int>> parent;   // producer -> (concat, float offset)
@@ -269,7 +277,7 @@ gboolean dR_planBuffers(dR_Graph* net) {
         if (n->type != tFullyConnected || (fuseFc && strcmp(fuseFc, "0") == 0)) continue;
         dR_FC_Data* fd = (dR_FC_Data*)n->layer;
         // an output node can defer too: its consumer stores the finished vector into its buffer
-        if (n->outputBuf || !n->next_layers || n->next_layers->length != 1) continue;
+        if (n->outputBuf || !n->next_layers || n->next_layers->length != 1 || n->layerID == g_debugLayerAtPlanTime) continue;
         if (drhip_fc_slices(fd->shape.s0, fd->shape.s1) <= 1) continue;
         dR_Node* c = nodes_of(n->next_layers)[0];
         if (c->type == tFullyConnected) ((dR_FC_Data*)c->layer)->drDeferredInput = n;

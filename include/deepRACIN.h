@@ -39,8 +39,12 @@ void       dR_config(dR_Graph* net, gchar* platformname, gboolean silent, gboole
 
 /* Bring up the device: selects HIP device clConfig->clDeviceNumber, creates the graph's stream.
  * Keeps its OpenCL-era name.  dR_prepare calls it implicitly if the caller did not.
- * (deepRACIN.h:155, deepRACIN.c:144) */
-void       dR_initCL(dR_Graph* net);
+ * Returns TRUE when the device is up.  The reference declares this function void (deepRACIN.h:155,
+ * deepRACIN.c:144-146), yet its own Python wrapper binds it with a bool result and refuses to go on when
+ * that is false (python/deepracin/__init__.py.in:55-58, 422-426): there the TRUE of dR_clInit happens to be
+ * left in the return register.  Here the result is returned on purpose; a C caller written against the
+ * void declaration ignores it. */
+gboolean   dR_initCL(dR_Graph* net);
 
 /* Mark a node whose buffer must survive dR_apply and be retrievable with dR_getOutputBuffers.
  * (deepRACIN.h:142, deepRACIN.c:133-141) */
@@ -55,8 +59,12 @@ gboolean   dR_prepare(dR_Graph* net);
  * owned by the graph and valid until dR_cleanup.  (deepRACIN.h:32, deepRACIN.c:51-72) */
 gint       dR_getOutputBuffers(dR_Graph* net, cl_mem** outptr);
 
-/* Blocking host->device copy of numfloats floats into the feed node's buffer, starting at float
- * index offset.  (deepRACIN.h:47, deepRACIN.c:74-77) */
+/* Host->device copy of numfloats floats into the feed node's buffer, starting at float index offset.
+ * The caller's array has been read when the call returns (it may be reused at once, as after the
+ * reference's blocking write); the transfer itself is asynchronous, from a pinned staging area the graph
+ * owns, ordered on the graph's stream in front of the next dR_apply.  Arrays larger than the staging area
+ * (sized at dR_prepare for the largest feed node) and DR_STAGING=0 take a blocking copy.
+ * (deepRACIN.h:47, deepRACIN.c:74-77) */
 void       dR_feedData(dR_Graph* net, dR_Node* feednode, gfloat* data, gint offset, gint numfloats);
 
 /* Enqueue one forward pass on the graph's stream; returns without waiting unless profiling is on.

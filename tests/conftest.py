@@ -1,3 +1,4 @@
+import ctypes
 import os
 import sys
 
@@ -40,6 +41,43 @@ def gpu(lib):
     rc = lib.drhip_init(0, info)
     assert rc == 0, "no usable gfx950 device: %s" % lib.drhip_last_error().decode()
     return info
+
+
+class Dev:
+    """Tiny RAII helper around drhip_malloc/upload/download for the tests."""
+
+    def __init__(self, lib):
+        self.lib = lib
+        self.ptrs = []
+
+    def put(self, arr):
+        arr = np.ascontiguousarray(arr)
+        p = ctypes.c_void_p()
+        assert self.lib.drhip_malloc(ctypes.byref(p), max(arr.nbytes, 4)) == 0, self.lib.drhip_last_error()
+        self.ptrs.append(p)
+        if arr.nbytes:
+            assert self.lib.drhip_upload(p, 0, arr.ctypes.data_as(ctypes.c_void_p), arr.nbytes, None) == 0
+        return p
+
+    def empty(self, n, dtype=np.float32):
+        return self.put(np.full(n, -777, dtype))       # poison: unwritten outputs are visible
+
+    def get(self, p, shape, dtype=np.float32):
+        out = np.empty(shape, dtype)
+        assert self.lib.drhip_download(out.ctypes.data_as(ctypes.c_void_p), p, 0, out.nbytes, None) == 0, self.lib.drhip_last_error()
+        return out
+
+    def close(self):
+        for p in self.ptrs:
+            self.lib.drhip_free(p)
+        self.ptrs = []
+
+
+@pytest.fixture
+def dev(lib, gpu):
+    d = Dev(lib)
+    yield d
+    d.close()
 
 
 def rel_err(a, b, floor=1e-30):

@@ -10,7 +10,7 @@ import os
 import numpy as np
 import pytest
 
-from conftest import assert_close, rel_err
+from conftest import Dev, assert_close, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -20,43 +20,6 @@ RNG = np.random.default_rng(7)
 
 def rnd(*shape, scale=1.0):
     return (RNG.standard_normal(shape) * scale).astype(np.float32)
-
-
-class Dev:
-    """Tiny RAII helper around drhip_malloc/upload/download for the tests."""
-
-    def __init__(self, lib):
-        self.lib = lib
-        self.ptrs = []
-
-    def put(self, arr):
-        arr = np.ascontiguousarray(arr)
-        p = ctypes.c_void_p()
-        assert self.lib.drhip_malloc(ctypes.byref(p), max(arr.nbytes, 4)) == 0, self.lib.drhip_last_error()
-        self.ptrs.append(p)
-        if arr.nbytes:
-            assert self.lib.drhip_upload(p, 0, arr.ctypes.data_as(ctypes.c_void_p), arr.nbytes, None) == 0
-        return p
-
-    def empty(self, n, dtype=np.float32):
-        return self.put(np.full(n, -777, dtype))       # poison: unwritten outputs are visible
-
-    def get(self, p, shape, dtype=np.float32):
-        out = np.empty(shape, dtype)
-        assert self.lib.drhip_download(out.ctypes.data_as(ctypes.c_void_p), p, 0, out.nbytes, None) == 0, self.lib.drhip_last_error()
-        return out
-
-    def close(self):
-        for p in self.ptrs:
-            self.lib.drhip_free(p)
-        self.ptrs = []
-
-
-@pytest.fixture
-def dev(lib, gpu):
-    d = Dev(lib)
-    yield d
-    d.close()
 
 
 def ok(lib, rc):

@@ -430,7 +430,7 @@ def test_second_prepare_is_refused_not_silently_empty(lib, capfd):
         capfd.readouterr()
         assert lib.dR_prepare(g.ptr) == 0
         out = capfd.readouterr().out
-        assert "prepared already" in out
+        assert "scheduled before" in out and "prepared already" not in out      # (scheduled by hand, never prepared)
         assert [dr.node_struct(n).drSchedulePos for n in nodes] == first
 
 
@@ -505,6 +505,35 @@ def test_layers_beyond_the_packed_argument_fields_take_the_general_kernel(lib):
             plan = plan_of(g, [c, p])
             if width > 65535:
                 assert plan[0][0] != plan[1][0]                  # the convolution keeps a tensor of its own
+
+
+def test_layers_beyond_32_bit_byte_offsets_take_the_general_kernels(lib):
+    """Every dimension fits the 16-bit argument fields, but the input holds 2^29 elements or more: the matrix-core
+    3x3 kernels and the pooling-on-load 1x1 kernel (32-bit byte offsets) are not scheduled for such a layer."""
+    rng = np.random.default_rng(0)
+    for width, bank in ((64, True), (65000, False)):
+        with dr.Environment() as env:                                         # strided 3x3: direct kernel, with or without its filter bank
+            g = env.create_graph()
+            x = dr.feed_node(g, [1033, width, 8])
+            c = dr.Conv2d_raw(x, rng.standard_normal((8, 2, 3, 3)), None, (2, 2), "relu")
+            dr.mark_as_output(c)
+            assert lib.dR_propagateShapesAndSchedule(g.ptr) == 1
+            line = _kernel_line(c)
+            assert "direct" in line and (("variant 0" not in line) == bank), line
+    class PoolData(ctypes.Structure):                                         # dR_Pooling_Data (include/dR_nodes.h)
+        _fields_ = [("ishape", ctypes.c_int * 3), ("shape", ctypes.c_int * 4), ("stride", ctypes.c_int * 4), ("poolingType", ctypes.c_int),
+                    ("shaderSrc", ctypes.c_void_p), ("useLMEM", ctypes.c_int), ("drFused", ctypes.c_int)]
+    for width, fused in ((64, True), (65000, False)):
+        with dr.Environment() as env:                                         # 3x3/2 max pool -> 1x1 conv
+            g = env.create_graph()
+            x = dr.feed_node(g, [1033, width, 8])
+            p = dr.Pooling(x, "max", [1, 3, 3, 1], [1, 2, 2, 1])
+            c = dr.Conv2d_raw(p, rng.standard_normal((8, 2, 1, 1)), None, (1, 1), "relu")
+            dr.mark_as_output(c)
+            assert lib.dR_propagateShapesAndSchedule(g.ptr) == 1
+            assert lib.dR_planBuffers(g.ptr) == 1
+            pd = ctypes.cast(dr.node_struct(p).layer, ctypes.POINTER(PoolData)).contents
+            assert bool(pd.drFused) == fused, (width, pd.drFused)
 
 
 def test_pick_variants_are_launchable(lib):
