@@ -102,13 +102,16 @@ KERNEL_NAMES = {"winograd": "winograd_f23_mfma_kernel", "conv1x1": "conv1x1_mfma
 def winograd_issued_flops(lib, W, H, I, O):
     """FLOPs the Winograd kernel issues for a layer: 16 GEMMs over tiles x I x O, each padded to the blocks of
     the variant the scheduler picks (tile blocks of 32 or 16, 8 input channels per stage, 32/64/128 or 16/32/64
-    output channels per workgroup)."""
+    output channels per workgroup); drhip_conv3x3_winograd_f32 decides the same way."""
     v = lib.drhip_conv3x3_winograd_pick_variant(W, H, I, O)
     tb = 16 if v & 0x100 else 32
     ob = tb * {1: 1, 2: 2, 3: 4}[v & 0xf]
     tiles = ((W + 1) // 2) * ((H + 1) // 2)
     pad = lambda n, m: -(-n // m) * m
-    return 2 * 16 * pad(tiles, tb) * pad(I, 8) * pad(O, ob)
+    # (an image layer -- at most 4 input channels, 32-tile blocks, unsplit, four waves -- runs its one stage without
+    # the two k-steps that would multiply zeros)
+    few = I <= 4 and tb == 32 and (v & 0xf) <= 2 and not (v & 0x400) and not (v >> 4) & 0xf
+    return 2 * 16 * pad(tiles, tb) * (4 if few else pad(I, 8)) * pad(O, ob)
 
 
 def measure(workload, seed, steps, warmup, blocks=BLOCKS, instrument=True, env_vars=None):

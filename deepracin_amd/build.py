@@ -85,5 +85,24 @@ def build(force=False, verbose=True):
     return LIB
 
 
+def build_c_caller(out=None, verbose=True):
+    """Compile tests/c_caller.c, a host program in plain C against the public headers (the shape of the reference's
+    own example program), with gcc and link it against the library.  Its _Static_assert block checks the struct
+    layouts of include/dR_types.h against the reference's (tests/golden/ref_struct_offsets.h)."""
+    tests = os.path.join(ROOT, "tests")
+    out = out or os.path.join(tests, "bin", "c_caller")
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    cmd = [os.environ.get("CC", "gcc"), "-std=c11", "-O1", "-Wall", "-Werror", "-I" + os.path.join(ROOT, "include"), "-I" + tests,
+           os.path.join(tests, "c_caller.c"), "-o", out, "-L" + LIBDIR, "-ldeepracin", "-Wl,-rpath," + LIBDIR,
+           "-Wl,-rpath,$ORIGIN/../../deepracin_amd/lib"]       # (found from tests/bin wherever the tree is copied to)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("compile failed: %s\n%s%s" % (" ".join(cmd), r.stdout, r.stderr))
+    if verbose:
+        print("built", out)
+    return out
+
+
 if __name__ == "__main__":
     build(force="--force" in sys.argv)
+    build_c_caller()

@@ -192,7 +192,9 @@ __device__ inline f32x4 buf_load4(__amdgpu_buffer_rsrc_t r, unsigned voffset, un
 // set 0 first.  One wave per SIMD cannot keep the matrix pipe busy (it waits for its own transforms and
 // loads); layers whose workgroup count leaves one workgroup per CU get their second wave per SIMD this way,
 // without a second workgroup's share of partial tiles in memory.
-template <int NT, int KW>
+// FEWC: a layer with at most four input channels (an image): one stage whose third and fourth k-step would multiply
+// zeros are left out, and nothing is prefetched.
+template <int NT, int KW, bool FEWC = false>
 __global__ void __launch_bounds__(kWinoThreads * KW, KW == 2 ? 1 : (NT == 1 ? 3 : (NT == 2 ? 2 : 1)))
 winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__ U, const float* __restrict__ bias,
                          WINO_ARGS, float* __restrict__ out, float* __restrict__ ws) {
@@ -317,10 +319,11 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[e][nt][r] = 0.0f;
 
+    constexpr int KS = FEWC ? 2 : 4;                // k-steps of a stage that carry channels
     float raw[4][8];
     f32x4 f[4][NT];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) load_rows_ranged(raw[ks], (chBegin + kset) * KC + 2 * ks);
+    for (int ks = 0; ks < KS; ++ks) load_rows_ranged(raw[ks], (chBegin + kset) * KC + 2 * ks);
 #pragma unroll
     for (int e = 0; e < 4; ++e) load_filters(f[e], e, min(chBegin + kset, nChunksAll - 1));
 
@@ -330,7 +333,7 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
         const int next = min(ch + KW, nChunksAll - 1);
         float b[4][4];                              // [k-step][xi within the row]
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < KS; ++ks) {
             float m[4];
 #pragma unroll
             for (int s = 0; s < 4; ++s) m[s] = fmaf(sgn, raw[ks][4 + s], raw[ks][s]);   // exact: sgn is +-1
@@ -352,12 +355,13 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
 #pragma unroll
         for (int eg = 0; eg < 2; ++eg) {
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
+            for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
                 for (int e = 2 * eg; e < 2 * eg + 2; ++e)
 #pragma unroll
                     for (int nt = 0; nt < NT; ++nt)
                         acc[e][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[e][nt][ks], b[ks][e], acc[e][nt], 0, 0, 0);
+                if constexpr (FEWC) continue;       // (a single stage: nothing to load for a next one)
                 if (eg == 0) {
                     if constexpr (decltype(plainNext)::value) load_rows_plain(raw[ks], (ch + KW) * KC + 2 * ks);
                     else load_rows_ranged(raw[ks], (ch + KW) * KC + 2 * ks);
@@ -367,8 +371,10 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        load_filters(f[2], 2, next);
-        load_filters(f[3], 3, next);
+        if constexpr (!FEWC) {
+            load_filters(f[2], 2, next);
+            load_filters(f[3], 3, next);
+        }
         __builtin_amdgcn_sched_barrier(0);
     };
     // Stages whose successor chunk (KW further on) is complete (all 8 channels exist) and does not hold the
@@ -898,9 +904,15 @@ static int launch_wino(const float* in, const float* U, const float* bias, float
                 launch((winograd_f23_mfma_kernel<NT, 2>), grid, dim3(2 * kWinoThreads), 2 * ldsBytes, s,
                        in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
         }
-        if (c.waveSets != 2 || NT > 2)
-            launch((winograd_f23_mfma_kernel<NT, 1>), grid, dim3(kWinoThreads), ldsBytes, s,
-                   in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
+        if (c.waveSets != 2 || NT > 2) {
+            if (NT <= 2 && I <= 4 && g.splits == 1) {       // an image: the stage without its two empty k-steps
+                if constexpr (NT <= 2)
+                    launch((winograd_f23_mfma_kernel<NT, 1, true>), grid, dim3(kWinoThreads), ldsBytes, s,
+                           in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
+            } else
+                launch((winograd_f23_mfma_kernel<NT, 1>), grid, dim3(kWinoThreads), ldsBytes, s,
+                       in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
+        }
     } else if (c.waveSets == 2)
         launch((winograd_f23_mfma16_kernel<NT, 2>), grid, dim3(2 * kWinoThreads), 2 * ldsBytes, s,
                in, U, bias, pa.wh, pa.io, pa.mulX, pa.mulTB, pa.cfg0, pa.cfg1, out, workspace);
@@ -960,13 +972,14 @@ extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
         return ((join && (nChunks >> lg) < 16) ? 0 : 0x400) | code | (lg << 4) | join;
     }
     // Unsplit layers with more 32-channel panels than CUs, but no multiple of them (112x112 128->128: 392 panels,
-    // two on 136 CUs and one on 120): tiers of whole, halved, ... panels even the CUs out (21.1 vs 23.2 us;
-    // 224x224 64->64: 22.7 vs 23.2 us).  With 8 stages and fewer than two whole panels per CU it is a tie.
+    // two on 136 CUs and one on 120): tiers of whole, halved, ... panels even the CUs out (in a replayed VGG16
+    // pass 18.4 vs 20.2 us, of which the layer behind it gives 0.5 us back).  With 8 stages it is a tie or a loss
+    // (224x224 64->64 as 32-channel panels in tiers: 20.4 vs 20.0 us for 64-channel panels).
     if (lg == 0 && wino_join_flag(1, 2)) {
         static const bool tiersOn = [] { const char* e = getenv("DR_WINO_TIERS"); return !(e && e[0] == '0'); }();
         const int cusPerXcd = cus / kXcds, P = ceil_div(ceil_div(T, 32) * ceil_div(O, 32), kXcds);
         WinoTiers t;
-        if (tiersOn && cusPerXcd > 0 && P >= cusPerXcd && P % cusPerXcd != 0 && (nChunks >= 16 || P >= 2 * cusPerXcd) &&
+        if (tiersOn && cusPerXcd > 0 && P >= cusPerXcd && P % cusPerXcd != 0 && nChunks >= 16 &&
             wino_tiers(ceil_div(T, 32) * ceil_div(O, 32), nChunks, cusPerXcd, &t))
             return 0x1801;
     }

@@ -285,3 +285,28 @@ def test_debug_layer_download_and_profiling_switches(lib, dev, oracle, capfd):
             assert lib.dR_apply(g.ptr)
             (soft,) = configs.fetch_chw(g)
             assert_close(soft.reshape(-1), want[4].reshape(-1), "softmax after the switches were turned off again")
+
+
+def test_compiled_c_host_program_classifies_the_reference_images(gpu, tmp_path):
+    """tests/c_caller.c, compiled with gcc against the public headers (by build(); compiled here if it is missing),
+    run as a child process: the reference example's sequence -- switches poked into net->config / net->clConfig,
+    dR_loadGraph of the stored SqueezeNet v1.1, feed / apply / download per image -- must name the classes the
+    reference documents for its two images (examples/squeezenet-v1.1/squeezenet_deployed.c:199-207)."""
+    import subprocess
+    from deepracin_amd import build
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "bin", "c_caller")
+    if not os.path.exists(exe):
+        exe = build.build_c_caller(verbose=False)
+    files = []
+    for name in ("tiger", "puzzle"):
+        img = np.load(os.path.join(GOLDEN, "%s_224_rgb_u8.npy" % name))
+        f = tmp_path / (name + ".f32")
+        np.ascontiguousarray(img.transpose(2, 0, 1).astype(np.float32)).tofile(str(f))
+        files.append(str(f))
+    r = subprocess.run([exe, os.path.join(GOLDEN, "squeezenet_whole") + "/", files[0], files[1], files[0]],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    classes = [int(l.split()[1]) for l in r.stdout.splitlines() if l.startswith("class ")]
+    assert classes == [292, 611, 292], r.stdout
+    assert "GPU Profiling: Sum of all kernel run times" in r.stdout and "CPU Profiling: Whole graph took" in r.stdout

@@ -536,6 +536,17 @@ def test_layers_beyond_32_bit_byte_offsets_take_the_general_kernels(lib):
             assert bool(pd.drFused) == fused, (width, pd.drFused)
 
 
+def test_c_host_program_compiles_against_the_public_headers(lib, tmp_path):
+    """tests/c_caller.c: plain C11 against include/deepRACIN.h, with one _Static_assert per field of the structs a
+    host program of the reference reaches into (offsets from the reference's own header, tests/golden/
+    ref_struct_offsets.h).  Compiling it is the layout check; it links against the library without a GPU."""
+    from deepracin_amd import build
+    exe = build.build_c_caller(out=str(tmp_path / "c_caller"), verbose=False)
+    import subprocess
+    r = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 2 and "usage" in r.stderr
+
+
 def test_pick_variants_are_launchable(lib):
     for (W, H, I, O) in [(224, 224, 3, 64), (224, 224, 64, 64), (56, 56, 256, 256), (14, 14, 512, 512), (55, 55, 16, 64), (1, 1, 1, 1)]:
         v = lib.drhip_conv3x3_winograd_pick_variant(W, H, I, O)

@@ -25,6 +25,14 @@ def _get(lib, p, n):
     return out
 
 
+def _free_device_bytes():
+    """hipMemGetInfo of the runtime the library itself is linked against (already loaded into this process)."""
+    hip = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert hip.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
 def test_fc_noalloc_matches_fc_on_two_calls_in_a_row(lib, gpu, oracle):
     rng = np.random.default_rng(2024)
     held = []
@@ -41,7 +49,11 @@ def test_fc_noalloc_matches_fc_on_two_calls_in_a_row(lib, gpu, oracle):
             y_ref, y_new = _put(lib, np.full(N, -777.0)), _put(lib, np.full(N, -555.0))
             held += [xd, Wd, bd, parts, y_ref, y_new]
             assert lib.drhip_fc_f32(xd, Wd, bd, y_ref, parts, K, N, relu, None) == 0, lib.drhip_last_error()
+            assert lib.drhip_stream_sync(None) == 0
+            free_before = _free_device_bytes()
             assert lib.drhip_fc_noalloc_f32(xd, Wd, bd, y_new, K, N, relu, None) == 0, lib.drhip_last_error()
+            assert lib.drhip_stream_sync(None) == 0
+            assert _free_device_bytes() == free_before, "device memory was taken or given back during the call"
             want, got = _get(lib, y_ref, N), _get(lib, y_new, N)
             assert np.array_equal(want, got), "K=%d N=%d: %d of %d elements differ" % (K, N, int((want != got).sum()), N)
             # and the existing entry point itself is right (oracle, 1e-4 of the layer's largest magnitude)
