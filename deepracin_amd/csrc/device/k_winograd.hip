@@ -241,286 +241,301 @@ winograd_f23_mfma_kernel(const float* __restrict__ in, const float* __restrict__
         else if (lgSp == 1) __builtin_amdgcn_s_setprio(1);
     }
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int waveId = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wave = waveId & 3;                    // = row of the transform
-    const int kset = waveId >> 2;                   // which of the KW wave sets
-    const int l32 = lane & 31, lhi = lane >> 5;
-    const int plane = H * W;
-    const int nChunksAll = (I + KC - 1) / KC;
-    const int chBegin = split * chunksHere;
-    const int chEnd = min(nChunksAll, chBegin + chunksHere);        // > chBegin: the launcher creates no empty split
-    const int Opad = wino_opad(O);
+    // With two wave sets the rest of the kernel exists twice, chosen once per workgroup: only the block that holds image
+    // tile 0 carries the three selects per k-step that move that one lane's samples (`shifted` below); in every other
+    // block they are constants and vanish.  (A branch inside the stage, and two copies of the channel loop alone, both cost more
+    // than they saved: the first breaks the stage's instruction order, the second made the compiler spill.)
+    auto rest_of_kernel = [&](auto tile0Block) {
+        const int tid = threadIdx.x, lane = tid & 63;
+        const int waveId = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int wave = waveId & 3;                    // = row of the transform
+        const int kset = waveId >> 2;                   // which of the KW wave sets
+        const int l32 = lane & 31, lhi = lane >> 5;
+        const int plane = H * W;
+        const int nChunksAll = (I + KC - 1) / KC;
+        const int chBegin = split * chunksHere;
+        const int chEnd = min(nChunksAll, chBegin + chunksHere);        // > chBegin: the launcher creates no empty split
+        const int Opad = wino_opad(O);
 
-    // ---- this lane's tile and the byte offsets of the two window rows it reads ---------------
-    // Row w of B^T d:  w=0: d0 - d2,  w=1: d1 + d2,  w=2: d2 - d1,  w=3: d3 - d1.
-    const int tg = t0 + l32;
-    const bool tileOk = tg < T;
-    const int ty = tileOk ? fast_div(tg, tilesXd) : 0, tx = tileOk ? tg - ty * tilesX : 0;
-    const int x0 = 2 * tx - 1, y0 = 2 * ty - 1;
-    const int rowA = wave, rowB = (wave < 2) ? 2 : 1;
-    const float sgn = (wave == 1) ? 1.0f : -1.0f;
-    // One 16-byte load per row from the (4-byte aligned) address of its first sample.  Rows outside
-    // the image carry the out-of-range offset as a whole; samples beyond the left or right edge come
-    // back as the neighbouring row's pixels and are zeroed by three selects after the rows have been
-    // combined (the second sample, x = 2*tx, always exists).  A negative offset would zero the whole
-    // load, and only image tile 0 has one (x = -1 in row 0): that one lane loads from x = 0 instead
-    // and shifts its combined samples up by one (three more selects for everybody; a branch around
-    // them costs more in register copies than it saves).
-    const bool shifted = tg == 0;
-    const int xLoad = shifted ? 0 : x0;
-    const int yaRow = y0 + rowA, ybRow = y0 + rowB;
-    const unsigned offVA = (tileOk && yaRow >= 0 && yaRow < H) ? 4u * (unsigned)(lhi * plane + yaRow * W + xLoad) : kOutOfRange;
-    const unsigned offVB = (tileOk && ybRow >= 0 && ybRow < H) ? 4u * (unsigned)(lhi * plane + ybRow * W + xLoad) : kOutOfRange;
-    const bool c0ok = x0 >= 0, c2ok = x0 + 2 < W, c3ok = x0 + 3 < W;
+        // ---- this lane's tile and the byte offsets of the two window rows it reads ---------------
+        // Row w of B^T d:  w=0: d0 - d2,  w=1: d1 + d2,  w=2: d2 - d1,  w=3: d3 - d1.
+        const int tg = t0 + l32;
+        const bool tileOk = tg < T;
+        const int ty = tileOk ? fast_div(tg, tilesXd) : 0, tx = tileOk ? tg - ty * tilesX : 0;
+        const int x0 = 2 * tx - 1, y0 = 2 * ty - 1;
+        const int rowA = wave, rowB = (wave < 2) ? 2 : 1;
+        const float sgn = (wave == 1) ? 1.0f : -1.0f;
+        // One 16-byte load per row from the (4-byte aligned) address of its first sample.  Rows outside
+        // the image carry the out-of-range offset as a whole; samples beyond the left or right edge come
+        // back as the neighbouring row's pixels and are zeroed by three selects after the rows have been
+        // combined (the second sample, x = 2*tx, always exists).  A negative offset would zero the whole
+        // load, and only image tile 0 has one (x = -1 in row 0): that one lane loads from x = 0 instead
+        // and shifts its combined samples up by one (three more selects for everybody; a branch around
+        // them costs more in register copies than it saves).
+        const bool shifted = decltype(tile0Block)::value && tg == 0;
+        const int xLoad = shifted ? 0 : x0;
+        const int yaRow = y0 + rowA, ybRow = y0 + rowB;
+        const unsigned offVA = (tileOk && yaRow >= 0 && yaRow < H) ? 4u * (unsigned)(lhi * plane + yaRow * W + xLoad) : kOutOfRange;
+        const unsigned offVB = (tileOk && ybRow >= 0 && ybRow < H) ? 4u * (unsigned)(lhi * plane + ybRow * W + xLoad) : kOutOfRange;
+        const bool c0ok = x0 >= 0, c2ok = x0 + 2 < W, c3ok = x0 + 3 < W;
+        const float k0f = c0ok ? 1.0f : 0.0f, k3f = c3ok ? 1.0f : 0.0f;
 
-    // Window rows of channels cbase + lhi.  "Ranged" form: the resource starts at channel cbase and
-    // ends with the tensor, so channels >= I read 0 without touching memory (ragged last chunk,
-    // prefetch past the end).  "Plain" form for chunks known to lie inside the tensor: one resource
-    // for the whole tensor, the channel offset travels in the scalar offset (a resource that changes
-    // inside the loop makes the compiler wait for all outstanding loads at the loop head).
-    const __amdgpu_buffer_rsrc_t rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kBufferFlags);
-    auto load_rows = [&](float (&d)[8], __amdgpu_buffer_rsrc_t r, unsigned soff) {
-        const f32x4 a = buf_load4(r, offVA, soff), b = buf_load4(r, offVB, soff);
+        // Window rows of channels cbase + lhi.  "Ranged" form: the resource starts at channel cbase and
+        // ends with the tensor, so channels >= I read 0 without touching memory (ragged last chunk,
+        // prefetch past the end).  "Plain" form for chunks known to lie inside the tensor: one resource
+        // for the whole tensor, the channel offset travels in the scalar offset (a resource that changes
+        // inside the loop makes the compiler wait for all outstanding loads at the loop head).
+        const __amdgpu_buffer_rsrc_t rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kBufferFlags);
+        auto load_rows = [&](float (&d)[8], __amdgpu_buffer_rsrc_t r, unsigned soff) {
+            const f32x4 a = buf_load4(r, offVA, soff), b = buf_load4(r, offVB, soff);
 #pragma unroll
-        for (int s = 0; s < 4; ++s) { d[s] = a[s]; d[4 + s] = b[s]; }
-    };
-    auto load_rows_plain = [&](float (&d)[8], int cbase) { load_rows(d, rIn, 4u * (unsigned)(cbase * plane)); };
-    auto load_rows_ranged = [&](float (&d)[8], int cbase) {
-        const int left = max(I - cbase, 0);
-        const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(in + (size_t)min(cbase, I) * plane), 0,
-                                                                             left * plane * 4, kBufferFlags);
-        load_rows(d, r, 0u);
-    };
-    // filters of one xi for a whole stage: component ks of the 16-byte load = k-step ks
-    const __amdgpu_buffer_rsrc_t rU = __builtin_amdgcn_make_buffer_rsrc((void*)U, 0, 16 * nChunksAll * Opad * 8 * 4, kBufferFlags);
-    const unsigned fOff = 4u * (unsigned)((o0 + l32) * 8 + 4 * lhi);
-    auto load_filters = [&](f32x4 (&f)[NT], int e, int chunk) {
-        const unsigned soff = 4u * (unsigned)(((4 * wave + e) * nChunksAll + chunk) * Opad * 8);
+            for (int s = 0; s < 4; ++s) { d[s] = a[s]; d[4 + s] = b[s]; }
+        };
+        auto load_rows_plain = [&](float (&d)[8], int cbase) { load_rows(d, rIn, 4u * (unsigned)(cbase * plane)); };
+        auto load_rows_ranged = [&](float (&d)[8], int cbase) {
+            const int left = max(I - cbase, 0);
+            const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void*)(in + (size_t)min(cbase, I) * plane), 0,
+                                                                                 left * plane * 4, kBufferFlags);
+            load_rows(d, r, 0u);
+        };
+        // filters of one xi for a whole stage: component ks of the 16-byte load = k-step ks
+        const __amdgpu_buffer_rsrc_t rU = __builtin_amdgcn_make_buffer_rsrc((void*)U, 0, 16 * nChunksAll * Opad * 8 * 4, kBufferFlags);
+        const unsigned fOff = 4u * (unsigned)((o0 + l32) * 8 + 4 * lhi);
+        auto load_filters = [&](f32x4 (&f)[NT], int e, int chunk) {
+            const unsigned soff = 4u * (unsigned)(((4 * wave + e) * nChunksAll + chunk) * Opad * 8);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) f[nt] = buf_load4(rU, fOff + 4u * (unsigned)(nt * 32 * 8), soff);
-    };
+            for (int nt = 0; nt < NT; ++nt) f[nt] = buf_load4(rU, fOff + 4u * (unsigned)(nt * 32 * 8), soff);
+        };
 
-    // The epilogue's bias values are fetched now: a load issued there would add a trip to memory
-    // to the tail of every workgroup.
-    constexpr bool kBiasEarly = NT <= 2;
-    constexpr int EO = 8 * KW;                      // output channels finished per pass of the epilogue
-    float biasEarly[kBiasEarly ? OB / EO : 1];
-    if (kBiasEarly && bias && (nSp == 1 || joined)) {
+        // The epilogue's bias values are fetched now: a load issued there would add a trip to memory
+        // to the tail of every workgroup.
+        constexpr bool kBiasEarly = NT <= 2;
+        constexpr int EO = 8 * KW;                      // output channels finished per pass of the epilogue
+        float biasEarly[kBiasEarly ? OB / EO : 1];
+        if (kBiasEarly && bias && (nSp == 1 || joined)) {
 #pragma unroll
-        for (int q = 0; q < OB / EO; ++q) biasEarly[q] = bias[min(o0 + (tid >> 5) + EO * q, O - 1)];
-    }
-
-    f32x16 acc[4][NT];
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[e][nt][r] = 0.0f;
-
-    constexpr int KS = FEWC ? 2 : 4;                // k-steps of a stage that carry channels
-    float raw[4][8];
-    f32x4 f[4][NT];
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) load_rows_ranged(raw[ks], (chBegin + kset) * KC + 2 * ks);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) load_filters(f[e], e, min(chBegin + kset, nChunksAll - 1));
-
-    // One stage: transform the rows of chunk ch (and start loading those of chunk ch+1 into the
-    // same registers), then 16*NT MFMAs, reloading the filters of each xi pair behind its MFMAs.
-    auto stage = [&](int ch, auto plainNext) {
-        const int next = min(ch + KW, nChunksAll - 1);
-        float b[4][4];                              // [k-step][xi within the row]
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            float m[4];
-#pragma unroll
-            for (int s = 0; s < 4; ++s) m[s] = fmaf(sgn, raw[ks][4 + s], raw[ks][s]);   // exact: sgn is +-1
-            const float s1 = shifted ? m[0] : m[1], s2 = shifted ? m[1] : m[2], s3 = shifted ? m[2] : m[3];
-            m[0] = c0ok ? m[0] : 0.0f;
-            m[1] = s1;
-            m[2] = c2ok ? s2 : 0.0f;
-            m[3] = c3ok ? s3 : 0.0f;
-            b[ks][0] = m[0] - m[2];
-            b[ks][1] = m[1] + m[2];
-            b[ks][2] = m[2] - m[1];
-            b[ks][3] = m[3] - m[1];
+            for (int q = 0; q < OB / EO; ++q) biasEarly[q] = bias[min(o0 + (tid >> 5) + EO * q, O - 1)];
         }
-        __builtin_amdgcn_sched_barrier(0);
-        // 8 slots of 2*NT MFMAs (two xi at a time: dependent MFMAs stay 2*NT apart).  The loads of
-        // the next stage are issued behind the MFMAs of a slot, so the matrix pipe keeps running
-        // while they go out: input rows in the first four slots (their registers are free since
-        // the transforms above), the filters of an xi pair once its last MFMA has been issued.
+
+        f32x16 acc[4][NT];
 #pragma unroll
-        for (int eg = 0; eg < 2; ++eg) {
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[e][nt][r] = 0.0f;
+
+        constexpr int KS = FEWC ? 2 : 4;                // k-steps of a stage that carry channels
+        float raw[4][8];
+        f32x4 f[4][NT];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) load_rows_ranged(raw[ks], (chBegin + kset) * KC + 2 * ks);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) load_filters(f[e], e, min(chBegin + kset, nChunksAll - 1));
+
+        // One stage: transform the rows of chunk ch (and start loading those of chunk ch+1 into the
+        // same registers), then 16*NT MFMAs, reloading the filters of each xi pair behind its MFMAs.
+        auto stage = [&](int ch, auto plainNext) {
+            const int next = min(ch + KW, nChunksAll - 1);
+            float b[4][4];                              // [k-step][xi within the row]
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
+                float m[4];
 #pragma unroll
-                for (int e = 2 * eg; e < 2 * eg + 2; ++e)
+                for (int s = 0; s < 4; ++s) m[s] = fmaf(sgn, raw[ks][4 + s], raw[ks][s]);   // exact: sgn is +-1
+                // (the masks of the first and fourth sample ride in the combinations: k0f and k3f are 1.0 or 0.0, so
+                // these are the same sums with one rounding, for two instructions less per k-step)
+                const float s1 = shifted ? m[0] : m[1], s2 = shifted ? m[1] : m[2], s3 = shifted ? m[2] : m[3];
+                const float t2 = c2ok ? s2 : 0.0f;
+                b[ks][0] = fmaf(k0f, m[0], -t2);
+                b[ks][1] = s1 + t2;
+                b[ks][2] = t2 - s1;
+                b[ks][3] = fmaf(k3f, s3, -s1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // 8 slots of 2*NT MFMAs (two xi at a time: dependent MFMAs stay 2*NT apart).  The loads of
+            // the next stage are issued behind the MFMAs of a slot, so the matrix pipe keeps running
+            // while they go out: input rows in the first four slots (their registers are free since
+            // the transforms above), the filters of an xi pair once its last MFMA has been issued.
 #pragma unroll
-                    for (int nt = 0; nt < NT; ++nt)
-                        acc[e][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[e][nt][ks], b[ks][e], acc[e][nt], 0, 0, 0);
-                if constexpr (FEWC) continue;       // (a single stage: nothing to load for a next one)
-                if (eg == 0) {
-                    if constexpr (decltype(plainNext)::value) load_rows_plain(raw[ks], (ch + KW) * KC + 2 * ks);
-                    else load_rows_ranged(raw[ks], (ch + KW) * KC + 2 * ks);
-                } else if (ks < 2) {
-                    load_filters(f[ks], ks, next);
+            for (int eg = 0; eg < 2; ++eg) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                    for (int e = 2 * eg; e < 2 * eg + 2; ++e)
+#pragma unroll
+                        for (int nt = 0; nt < NT; ++nt)
+                            acc[e][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(f[e][nt][ks], b[ks][e], acc[e][nt], 0, 0, 0);
+                    if constexpr (FEWC) continue;       // (a single stage: nothing to load for a next one)
+                    if (eg == 0) {
+                        if constexpr (decltype(plainNext)::value) load_rows_plain(raw[ks], (ch + KW) * KC + 2 * ks);
+                        else load_rows_ranged(raw[ks], (ch + KW) * KC + 2 * ks);
+                    } else if (ks < 2) {
+                        load_filters(f[ks], ks, next);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (!FEWC) {
+                load_filters(f[2], 2, next);
+                load_filters(f[3], 3, next);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        // Stages whose successor chunk (KW further on) is complete (all 8 channels exist) and does not hold the
+        // tensor's last channel prefetch in the plain form; the last ones of the tensor use the ranged form.  (The
+        // scalar offset of a buffer access is not part of its range check, and the 16-byte row loads of the last
+        // tiles of the last row reach one or two samples past the row: in the last channel that is past the tensor,
+        // where only the ranged form's resource ends.)
+        const int chMain = min(chEnd, (I - 1) / KC - KW);
+        int ch = chBegin + kset;
+        for (; ch < chMain; ch += KW) stage(ch, std::true_type{});
+        for (; ch < chEnd; ch += KW) stage(ch, std::false_type{});
+
+        // ---- epilogue -----------------------------------------------------------------------------
+        // Accumulator layout of the 32x32 MFMA: lane -> column (tile) lane%32; register r -> row
+        // (output channel) 8*(r/4) + 4*(lane/32) + r%4.
+        // Each wave applies the right factor A to its row of M and parks the two results per
+        // (tile, channel) in LDS: P[row][j][channel][tile].
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float m0 = acc[0][nt][r], m1 = acc[1][nt][r], m2 = acc[2][nt][r], m3 = acc[3][nt][r];
+                const int ol = 32 * nt + 8 * (r / 4) + 4 * lhi + (r % 4);
+                P[(((kset * 4 + wave) * 2 + 0) * OB + ol) * TB + l32] = m0 + m1 + m2;
+                P[(((kset * 4 + wave) * 2 + 1) * OB + ol) * TB + l32] = m1 - m2 + m3;
             }
         }
-        if constexpr (!FEWC) {
-            load_filters(f[2], 2, next);
-            load_filters(f[3], 3, next);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    // Stages whose successor chunk (KW further on) is complete (all 8 channels exist) and does not hold the
-    // tensor's last channel prefetch in the plain form; the last ones of the tensor use the ranged form.  (The
-    // scalar offset of a buffer access is not part of its range check, and the 16-byte row loads of the last
-    // tiles of the last row reach one or two samples past the row: in the last channel that is past the tensor,
-    // where only the ranged form's resource ends.)
-    const int chMain = min(chEnd, (I - 1) / KC - KW);
-    int ch = chBegin + kset;
-    for (; ch < chMain; ch += KW) stage(ch, std::true_type{});
-    for (; ch < chEnd; ch += KW) stage(ch, std::false_type{});
+        // LDS-only barrier: __syncthreads() would also wait for the outstanding (unused) prefetches.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 
-    // ---- epilogue -----------------------------------------------------------------------------
-    // Accumulator layout of the 32x32 MFMA: lane -> column (tile) lane%32; register r -> row
-    // (output channel) 8*(r/4) + 4*(lane/32) + r%4.
-    // Each wave applies the right factor A to its row of M and parks the two results per
-    // (tile, channel) in LDS: P[row][j][channel][tile].
+        // Left factor A^T over the four rows, bias, ReLU, store: lane -> tile tid%32, channels tid/32 + EO*q.
+        const bool direct = nSp == 1;
+        const int et = tid & 31, eo = tid >> 5;
+        const int etg = t0 + et;
+        const bool eTileOk = etg < T;
+        const int eTy = eTileOk ? fast_div(etg, tilesXd) : 0;
+        const int ox = eTileOk ? 2 * (etg - eTy * tilesX) : 0, oy = 2 * eTy;
+        f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
+        // this lane's 2x2 tile of channel ol, summed over the rows of the transform (and the wave sets)
+        auto tile_of = [&](int ol) {
+            float p[4][2];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const float m0 = acc[0][nt][r], m1 = acc[1][nt][r], m2 = acc[2][nt][r], m3 = acc[3][nt][r];
-            const int ol = 32 * nt + 8 * (r / 4) + 4 * lhi + (r % 4);
-            P[(((kset * 4 + wave) * 2 + 0) * OB + ol) * TB + l32] = m0 + m1 + m2;
-            P[(((kset * 4 + wave) * 2 + 1) * OB + ol) * TB + l32] = m1 - m2 + m3;
-        }
-    }
-    // LDS-only barrier: __syncthreads() would also wait for the outstanding (unused) prefetches.
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-
-    // Left factor A^T over the four rows, bias, ReLU, store: lane -> tile tid%32, channels tid/32 + EO*q.
-    const bool direct = nSp == 1;
-    const int et = tid & 31, eo = tid >> 5;
-    const int etg = t0 + et;
-    const bool eTileOk = etg < T;
-    const int eTy = eTileOk ? fast_div(etg, tilesXd) : 0;
-    const int ox = eTileOk ? 2 * (etg - eTy * tilesX) : 0, oy = 2 * eTy;
-    f32x4* wsTiles = direct ? nullptr : (f32x4*)ws + ((size_t)split * nBlocks + logical) * OB * TB;
-    // this lane's 2x2 tile of channel ol, summed over the rows of the transform (and the wave sets)
-    auto tile_of = [&](int ol) {
-        float p[4][2];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            p[r][0] = P[((r * 2 + 0) * OB + ol) * TB + et];
-            p[r][1] = P[((r * 2 + 1) * OB + ol) * TB + et];
-            if constexpr (KW == 2) {                // the second wave set's half of the channel sum
-                p[r][0] += P[(((4 + r) * 2 + 0) * OB + ol) * TB + et];
-                p[r][1] += P[(((4 + r) * 2 + 1) * OB + ol) * TB + et];
+            for (int r = 0; r < 4; ++r) {
+                p[r][0] = P[((r * 2 + 0) * OB + ol) * TB + et];
+                p[r][1] = P[((r * 2 + 1) * OB + ol) * TB + et];
+                if constexpr (KW == 2) {                // the second wave set's half of the channel sum
+                    p[r][0] += P[(((4 + r) * 2 + 0) * OB + ol) * TB + et];
+                    p[r][1] += P[(((4 + r) * 2 + 1) * OB + ol) * TB + et];
+                }
             }
-        }
-        return f32x4{p[0][0] + p[1][0] + p[2][0], p[0][1] + p[1][1] + p[2][1],
-                     p[1][0] - p[2][0] + p[3][0], p[1][1] - p[2][1] + p[3][1]};
-    };
-    if (joined && nSp > 1) {
-        // (the partial tiles go out and are looked for at the highest priority: the other workgroups on this CU
-        // are in their channel loops, and a wave at their priority gets an issue slot only when they stall)
-        if (tiered) __builtin_amdgcn_s_setprio(3);
-        // Every split finishes the channels ol with ol >> lgRows == split of its panel (OB >> lgSplits channels).
-        // First the partial tiles the other splits are waiting for go out, written through; then this split
-        // collects theirs.  A workspace slot holds kWinoEmpty (a signalling NaN, which no addition can produce)
-        // until its partial tile has been stored, so a reader sees from the slot itself whether the data has
-        // arrived: no flag, no counter, no wait for the stores to complete.  The reader puts kWinoEmpty back.
-        const int lgRows = __builtin_ctz(OB) - lgSp;
-        const __amdgpu_buffer_rsrc_t rWs = __builtin_amdgcn_make_buffer_rsrc((void*)ws, 0, 0x7ffffff0, kBufferFlags);
-        const unsigned panelFloats = (unsigned)(OB * TB * 4);
-        // (tiered: a workgroup's partial tiles lie at its own index in the grid, its partners' 8 workgroups apart)
-        const unsigned region0 = tiered ? blockIdx.x - (unsigned)(kXcds * split) : (unsigned)logical;
-        const unsigned regionStep = tiered ? (unsigned)kXcds : (unsigned)nBlocks;
-        // byte address of a slot = region of the split (scalar offset) + place of the tile in the panel (per lane)
-        auto region_of = [&](int sp) { return (int)(4u * (region0 + (unsigned)sp * regionStep) * panelFloats); };
-        auto place_of = [&](int ol) { return (int)(16u * (unsigned)(ol * TB + et)); };
-#pragma unroll
-        for (int q = 0; q < OB / EO; ++q) {
-            const int ol = eo + EO * q;
-            if ((ol >> lgRows) == split) continue;
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, tile_of(ol)), rWs, place_of(ol), region_of(split), kAuxThrough);
-        }
-        const u32x4 empty = {kWinoEmpty, kWinoEmpty, kWinoEmpty, kWinoEmpty};
-        // (the number of splits as a constant: every access below is unconditional.  The slot of the own split is
-        // read and reset like the others - nobody ever writes it - and its content replaced by the own tile.)
-        auto collect = [&](auto nSplitsConst) {
-            constexpr int S = decltype(nSplitsConst)::value;
+            return f32x4{p[0][0] + p[1][0] + p[2][0], p[0][1] + p[1][1] + p[2][1],
+                         p[1][0] - p[2][0] + p[3][0], p[1][1] - p[2][1] + p[3][1]};
+        };
+        if (joined && nSp > 1) {
+            // (the partial tiles go out and are looked for at the highest priority: the other workgroups on this CU
+            // are in their channel loops, and a wave at their priority gets an issue slot only when they stall)
+            if (tiered) __builtin_amdgcn_s_setprio(3);
+            // Every split finishes the channels ol with ol >> lgRows == split of its panel (OB >> lgSplits channels).
+            // First the partial tiles the other splits are waiting for go out, written through; then this split
+            // collects theirs.  A workspace slot holds kWinoEmpty (a signalling NaN, which no addition can produce)
+            // until its partial tile has been stored, so a reader sees from the slot itself whether the data has
+            // arrived: no flag, no counter, no wait for the stores to complete.  The reader puts kWinoEmpty back.
+            const int lgRows = __builtin_ctz(OB) - lgSp;
+            const __amdgpu_buffer_rsrc_t rWs = __builtin_amdgcn_make_buffer_rsrc((void*)ws, 0, 0x7ffffff0, kBufferFlags);
+            const unsigned panelFloats = (unsigned)(OB * TB * 4);
+            // (tiered: a workgroup's partial tiles lie at its own index in the grid, its partners' 8 workgroups apart)
+            const unsigned region0 = tiered ? blockIdx.x - (unsigned)(kXcds * split) : (unsigned)logical;
+            const unsigned regionStep = tiered ? (unsigned)kXcds : (unsigned)nBlocks;
+            // byte address of a slot = region of the split (scalar offset) + place of the tile in the panel (per lane)
+            auto region_of = [&](int sp) { return (int)(4u * (region0 + (unsigned)sp * regionStep) * panelFloats); };
+            auto place_of = [&](int ol) { return (int)(16u * (unsigned)(ol * TB + et)); };
 #pragma unroll
             for (int q = 0; q < OB / EO; ++q) {
-                const int ol = eo + EO * q, o = o0 + ol;
-                if ((ol >> lgRows) != split) continue;
-                const f32x4 own = tile_of(ol);
-                u32x4 part[S];
-                bool ready = false;
-                for (int spins = 0; spins < kWinoJoinSpins && !ready; ++spins) {
-                    // (the loads are invariant as far as the compiler can see: without this it issues them once,
-                    // in front of the loop)
-                    asm volatile("" ::: "memory");
-                    ready = true;
-#pragma unroll
-                    for (int u = 0; u < S; ++u) part[u] = __builtin_amdgcn_raw_buffer_load_b128(rWs, place_of(ol), region_of(u), kAuxDeviceVolatile);
-#pragma unroll
-                    for (int u = 0; u < S; ++u)
-                        ready = ready && (u == split || (part[u][0] != kWinoEmpty && part[u][1] != kWinoEmpty && part[u][2] != kWinoEmpty && part[u][3] != kWinoEmpty));
-                }
-                f32x4 s = {0.f, 0.f, 0.f, 0.f};     // splits added in order, like winograd_split_reduce_kernel
-#pragma unroll
-                for (int u = 0; u < S; ++u) s += (u == split) ? own : __builtin_bit_cast(f32x4, part[u]);
-#pragma unroll
-                for (int u = 0; u < S; ++u) __builtin_amdgcn_raw_buffer_store_b128(empty, rWs, place_of(ol), region_of(u), kAuxThrough);
-                if (!ready) {                       // a partner never delivered: say so in the result and in the counter
-                    s = f32x4{__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
-                    atomicAdd(&g_wino_join_timeouts, 1u);
-                }
-                if (eTileOk && o < O) {
-                    if (bias) s += kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o];
-                    if (relu & kEpiRelu) { s[0] = fmaxf(s[0], 0.f); s[1] = fmaxf(s[1], 0.f); s[2] = fmaxf(s[2], 0.f); s[3] = fmaxf(s[3], 0.f); }
-                    if (relu & kEpiMaxPool2)
-                        store1_through(out + (size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
-                    else
-                        wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, s[0], s[1], s[2], s[3]);
-                }
+                const int ol = eo + EO * q;
+                if ((ol >> lgRows) == split) continue;
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, tile_of(ol)), rWs, place_of(ol), region_of(split), kAuxThrough);
             }
-        };
-        static_assert(kWinoMaxJoin == 16, "the cases below");
-        if (lgSp == 1) collect(std::integral_constant<int, 2>{});
-        else if (lgSp == 2) collect(std::integral_constant<int, 4>{});
-        else if (lgSp == 3) collect(std::integral_constant<int, 8>{});
-        else collect(std::integral_constant<int, 16>{});
-        return;
-    }
+            const u32x4 empty = {kWinoEmpty, kWinoEmpty, kWinoEmpty, kWinoEmpty};
+            // (the number of splits as a constant: every access below is unconditional.  The slot of the own split is
+            // read and reset like the others - nobody ever writes it - and its content replaced by the own tile.)
+            auto collect = [&](auto nSplitsConst) {
+                constexpr int S = decltype(nSplitsConst)::value;
 #pragma unroll
-    for (int q = 0; q < OB / EO; ++q) {
-        const int ol = eo + EO * q, o = o0 + ol;
-        const f32x4 y = tile_of(ol);
-        float y00 = y[0], y01 = y[1], y10 = y[2], y11 = y[3];
-        if (direct) {
-            if (eTileOk && o < O) {
-                if (bias) { const float bv = kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
-                if (relu & kEpiRelu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
-                if (relu & kEpiMaxPool2)        // W, H even: the tile is one window of a 2x2/2 max pool
-                    store1_through(out + (size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(y00, y01), fmaxf(y10, y11)));
-                else
-                    wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, y00, y01, y10, y11);
-            }
-        } else {
-            f32x4 v = {y00, y01, y10, y11};
-            wsTiles[(size_t)ol * TB + et] = v;      // whole panel, padding included: 512 B per half wave
+                for (int q = 0; q < OB / EO; ++q) {
+                    const int ol = eo + EO * q, o = o0 + ol;
+                    if ((ol >> lgRows) != split) continue;
+                    const f32x4 own = tile_of(ol);
+                    u32x4 part[S];
+                    bool ready = false;
+                    for (int spins = 0; spins < kWinoJoinSpins && !ready; ++spins) {
+                        // (the loads are invariant as far as the compiler can see: without this it issues them once,
+                        // in front of the loop)
+                        asm volatile("" ::: "memory");
+                        ready = true;
+#pragma unroll
+                        for (int u = 0; u < S; ++u) part[u] = __builtin_amdgcn_raw_buffer_load_b128(rWs, place_of(ol), region_of(u), kAuxDeviceVolatile);
+#pragma unroll
+                        for (int u = 0; u < S; ++u)
+                            ready = ready && (u == split || (part[u][0] != kWinoEmpty && part[u][1] != kWinoEmpty && part[u][2] != kWinoEmpty && part[u][3] != kWinoEmpty));
+                    }
+                    f32x4 s = {0.f, 0.f, 0.f, 0.f};     // splits added in order, like winograd_split_reduce_kernel
+#pragma unroll
+                    for (int u = 0; u < S; ++u) s += (u == split) ? own : __builtin_bit_cast(f32x4, part[u]);
+#pragma unroll
+                    for (int u = 0; u < S; ++u) __builtin_amdgcn_raw_buffer_store_b128(empty, rWs, place_of(ol), region_of(u), kAuxThrough);
+                    if (!ready) {                       // a partner never delivered: say so in the result and in the counter
+                        s = f32x4{__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
+                        atomicAdd(&g_wino_join_timeouts, 1u);
+                    }
+                    if (eTileOk && o < O) {
+                        if (bias) s += kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o];
+                        if (relu & kEpiRelu) { s[0] = fmaxf(s[0], 0.f); s[1] = fmaxf(s[1], 0.f); s[2] = fmaxf(s[2], 0.f); s[3] = fmaxf(s[3], 0.f); }
+                        if (relu & kEpiMaxPool2)
+                            store1_through(out + (size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+                        else
+                            wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, s[0], s[1], s[2], s[3]);
+                    }
+                }
+            };
+            static_assert(kWinoMaxJoin == 16, "the cases below");
+            if (lgSp == 1) collect(std::integral_constant<int, 2>{});
+            else if (lgSp == 2) collect(std::integral_constant<int, 4>{});
+            else if (lgSp == 3) collect(std::integral_constant<int, 8>{});
+            else collect(std::integral_constant<int, 16>{});
+            return;
         }
+#pragma unroll
+        for (int q = 0; q < OB / EO; ++q) {
+            const int ol = eo + EO * q, o = o0 + ol;
+            const f32x4 y = tile_of(ol);
+            float y00 = y[0], y01 = y[1], y10 = y[2], y11 = y[3];
+            if (direct) {
+                if (eTileOk && o < O) {
+                    if (bias) { const float bv = kBiasEarly ? biasEarly[kBiasEarly ? q : 0] : bias[o]; y00 += bv; y01 += bv; y10 += bv; y11 += bv; }
+                    if (relu & kEpiRelu) { y00 = fmaxf(y00, 0.f); y01 = fmaxf(y01, 0.f); y10 = fmaxf(y10, 0.f); y11 = fmaxf(y11, 0.f); }
+                    if (relu & kEpiMaxPool2)        // W, H even: the tile is one window of a 2x2/2 max pool
+                        store1_through(out + (size_t)o * (plane >> 2) + (size_t)(oy >> 1) * (W >> 1) + (ox >> 1), fmaxf(fmaxf(y00, y01), fmaxf(y10, y11)));
+                    else
+                        wino_store_tile(out + (size_t)o * plane + (size_t)oy * W + ox, W, H, ox, oy, vec2, y00, y01, y10, y11);
+                }
+            } else {
+                f32x4 v = {y00, y01, y10, y11};
+                wsTiles[(size_t)ol * TB + et] = v;      // whole panel, padding included: 512 B per half wave
+            }
+        }
+    };
+    // (Only the eight-wave form pays back the second copy: the first layers' kernels are so short that fetching
+    // twice the code costs them more - 224x224 3->64: 7.7-8.9 against 6.9 us - and the 32-channel four-wave form
+    // gained nothing.)
+    if constexpr (KW == 2) {
+        if (t0 == 0) rest_of_kernel(std::true_type{});
+        else rest_of_kernel(std::false_type{});
+    } else {
+        rest_of_kernel(std::true_type{});
     }
 }
 
@@ -579,6 +594,7 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
     const unsigned offVA = (tileOk && yaRow >= 0 && yaRow < H) ? 4u * (unsigned)(lk * plane + yaRow * W + xLoad) : kOutOfRange;
     const unsigned offVB = (tileOk && ybRow >= 0 && ybRow < H) ? 4u * (unsigned)(lk * plane + ybRow * W + xLoad) : kOutOfRange;
     const bool c0ok = x0 >= 0, c2ok = x0 + 2 < W, c3ok = x0 + 3 < W;
+    const float k0f = c0ok ? 1.0f : 0.0f, k3f = c3ok ? 1.0f : 0.0f;
 
     const __amdgpu_buffer_rsrc_t rIn = __builtin_amdgcn_make_buffer_rsrc((void*)in, 0, I * plane * 4, kBufferFlags);
     auto load_rows = [&](float (&d)[8], __amdgpu_buffer_rsrc_t r, unsigned soff) {
@@ -631,15 +647,14 @@ winograd_f23_mfma16_kernel(const float* __restrict__ in, const float* __restrict
             float m[4];
 #pragma unroll
             for (int s = 0; s < 4; ++s) m[s] = fmaf(sgn, raw[ks][4 + s], raw[ks][s]);
+            // (the masks of the first and fourth sample ride in the combinations: k0f and k3f are 1.0 or 0.0, so
+            // these are the same sums with one rounding, for two instructions less per k-step)
             const float s1 = shifted ? m[0] : m[1], s2 = shifted ? m[1] : m[2], s3 = shifted ? m[2] : m[3];
-            m[0] = c0ok ? m[0] : 0.0f;
-            m[1] = s1;
-            m[2] = c2ok ? s2 : 0.0f;
-            m[3] = c3ok ? s3 : 0.0f;
-            b[ks][0] = m[0] - m[2];
-            b[ks][1] = m[1] + m[2];
-            b[ks][2] = m[2] - m[1];
-            b[ks][3] = m[3] - m[1];
+            const float t2 = c2ok ? s2 : 0.0f;
+            b[ks][0] = fmaf(k0f, m[0], -t2);
+            b[ks][1] = s1 + t2;
+            b[ks][2] = t2 - s1;
+            b[ks][3] = fmaf(k3f, s3, -s1);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
