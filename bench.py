@@ -23,7 +23,11 @@ of 20 passes is a few milliseconds long and a single sample of it says little), 
                  `mfma_busy_frac_counters` is the same share from SQ_VALU_MFMA_BUSY_CYCLES of the
                  committed rocprofv3 run (profiles/counters.json: busy cycles per SIMD / (this run's device
                  time x 2.4 GHz)), `mfma_busy_frac_profiled` the share over the profiler's own, longer,
-                 kernel durations; null when there is no such run.  Device
+                 kernel durations; null when there is no such run (or when profiles/counters.json was written for
+                 other kernel sources).  `mfma_stream_clock_mhz` = the shader clock under a stream of fp32 MFMAs,
+                 measured in this run (drhip_mfma_clock_probe): the data-sheet peak assumes 2400 MHz, so
+                 `mfma_busy_frac_at_stream_clock` = mfma_busy_frac x 2400 / that clock is the share of the matrix
+                 cycles the part really offers under such load.  Device
                  times come from HIP events on the graph's own stream in a separate instrumented region:
                  with profilingGPU set the library attaches a start and a stop event to every kernel
                  launch, so a launch's span is the kernel alone, as in a rocprofv3 kernel trace.
@@ -296,7 +300,7 @@ def compact_roofline(r):
     if not r:
         return r
     keep = ("kernel", "bound", "achieved", "peak", "unit", "frac", "frac_issued", "traffic", "mfma_busy_frac_counters",
-            "mfma_busy_frac_profiled", "launches_per_step", "avg_launch_ms")
+            "mfma_busy_frac_profiled", "mfma_stream_clock_mhz", "mfma_busy_frac_at_stream_clock", "launches_per_step", "avg_launch_ms")
     return {k: r[k] for k in keep if k in r}
 
 
@@ -531,6 +535,15 @@ def main():
     m = measure(args.workload, args.seed, args.steps, args.warmup, args.blocks)
     spec, feeds, flops = m["spec"], m["feeds"], m["flops"]
     layers, groups, roofline, roofline_fc = analyse(lib, m, args.workload, counters)
+
+    # The data-sheet matrix peak is quoted at 2.4 GHz; under a stream of fp32 MFMAs the part runs slower (power).  The
+    # clock of such a stream, measured now on this GPU, caps every utilisation figure against the data-sheet peak.
+    mhz, probe_us = ctypes.c_float(0.0), ctypes.c_float(0.0)
+    lib.drhip_mfma_clock_probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
+    if lib.drhip_mfma_clock_probe(200, 500, ctypes.byref(mhz), ctypes.byref(probe_us), None) == 0 and mhz.value > 0 and roofline and "mfma_busy_frac" in roofline:
+        roofline["mfma_stream_clock_mhz"] = round(mhz.value, 1)
+        roofline["mfma_stream_probe_us"] = round(probe_us.value, 1)
+        roofline["mfma_busy_frac_at_stream_clock"] = round(roofline["mfma_busy_frac"] * PEAK_CLOCK_GHZ * 1e3 / mhz.value, 4)
 
     secondary = None
     other = {"vgg16": "squeezenet", "squeezenet": "vgg16"}.get(args.workload)

@@ -2,6 +2,9 @@
 #include "drhip_common.hpp"
 
 #include <algorithm>
+#include <vector>
+
+#include <algorithm>
 #include <chrono>
 #include <cstdlib>
 #include <cstring>
@@ -56,11 +59,64 @@ __global__ void __launch_bounds__(256) copy_from_host_kernel(float* __restrict__
     if (blockIdx.x == 0 && threadIdx.x < n - 4 * n4) dst[4 * n4 + threadIdx.x] = src[4 * n4 + threadIdx.x];
 }
 
+// Measurement aid: what the shader clock does under a stream of fp32 MFMAs.  Every wave issues `iters` rounds of 8
+// independent v_mfma_f32_32x32x2_f32 and reads the shader-clock counter (s_memtime) and the constant 100 MHz
+// counter (s_memrealtime) in front of and behind them; ticks[2 * wave] / ticks[2 * wave + 1] = clock / 100 MHz.
+typedef float f32x16p __attribute__((ext_vector_type(16)));
+__global__ void __launch_bounds__(256) mfma_clock_probe_kernel(long long* __restrict__ ticks, int iters, float seed) {
+    f32x16p acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = 0.f;
+    const float a = seed + threadIdx.x, b = seed * 0.5f;
+    const long long c0 = clock64(), w0 = wall_clock64();
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sum += acc[i][0] + acc[i][9];
+    const long long c1 = clock64(), w1 = wall_clock64();
+    if ((threadIdx.x & 63) == 0) {
+        const size_t wave = (size_t)blockIdx.x * (blockDim.x / 64) + threadIdx.x / 64;
+        ticks[2 * wave] = (c1 - c0) + (sum == 12345.678f ? 1 : 0);     // (keeps the arithmetic alive)
+        ticks[2 * wave + 1] = w1 - w0;
+    }
+}
+
 }  // namespace drhip
 
 using namespace drhip;
 
 extern "C" {
+
+int drhip_mfma_clock_probe(int iters, int launches, float* mhz_median, float* microseconds, void* stream) {
+    DRHIP_REQUIRE(iters > 0 && iters <= (1 << 20) && launches > 0 && launches <= (1 << 16) && mhz_median, "drhip_mfma_clock_probe: bad arguments");
+    const int wgs = 2 * num_cu(), waves = wgs * 4;
+    long long* d = nullptr;
+    if (int rc = check(hipMalloc((void**)&d, sizeof(long long) * 2 * waves), "hipMalloc(clock probe)")) return rc;
+    std::vector<long long> h(2 * (size_t)waves);
+    int rc = DRHIP_OK;
+    for (int rep = 0; rep < launches && rc == DRHIP_OK; ++rep) {   // back to back; the last launch is the one that is read
+        launch(mfma_clock_probe_kernel, dim3(wgs), dim3(256), 0, as_stream(stream), d, iters, 1.0f);
+        rc = launched("mfma_clock_probe_kernel");
+    }
+    if (rc == DRHIP_OK) rc = check(hipMemcpyAsync(h.data(), d, sizeof(long long) * h.size(), hipMemcpyDeviceToHost, as_stream(stream)), "hipMemcpyAsync(clock probe)");
+    if (rc == DRHIP_OK) rc = check(hipStreamSynchronize(as_stream(stream)), "hipStreamSynchronize(clock probe)");
+    (void)hipFree(d);
+    if (rc != DRHIP_OK) return rc;
+    std::vector<double> mhz, us;
+    for (int w = 0; w < waves; ++w)
+        if (h[2 * w + 1] > 0) { mhz.push_back(100.0 * (double)h[2 * w] / (double)h[2 * w + 1]); us.push_back((double)h[2 * w + 1] / 100.0); }
+    DRHIP_REQUIRE(!mhz.empty(), "drhip_mfma_clock_probe: the probe recorded nothing");
+    std::sort(mhz.begin(), mhz.end());
+    std::sort(us.begin(), us.end());
+    *mhz_median = (float)mhz[mhz.size() / 2];
+    if (microseconds) *microseconds = (float)us[us.size() / 2];
+    return DRHIP_OK;
+}
 
 const char* drhip_last_error(void) { return error_slot(); }
 

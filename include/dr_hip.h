@@ -67,6 +67,14 @@ int drhip_timing_begin(void);
 int drhip_timing_count(void);
 int drhip_timing_end(float* ms, int capacity, int* count);
 int drhip_stream_wait_event(void* stream, void* ev);      /* later work on `stream` starts after `ev`; joins a capture */
+/* Measurement aid (no counterpart in the reference): the shader clock under a stream of fp32 MFMAs.  Two workgroups
+ * per CU issue `iters` rounds of 8 independent v_mfma_f32_32x32x2_f32 per wave and read the shader-clock counter and
+ * the constant 100 MHz counter around them; the kernel is launched `launches` times back to back (power management
+ * reacts over milliseconds: a single short launch still sees idle clocks) and the last launch is read:
+ * *mhz_median = median over its waves of the counters' ratio x 100 MHz, *microseconds (may be NULL) = median
+ * duration of the measured stretch.  The data-sheet peak of the matrix cores
+ * is quoted at 2400 MHz; utilisation figures against that peak are capped by this ratio.  Allocates and blocks. */
+int drhip_mfma_clock_probe(int iters, int launches, float* mhz_median, float* microseconds, void* stream);
 
 /* ---- launch graphs: record everything enqueued on `stream` between begin and end into an executable
  *      hipGraph and replay it with one call.  Used by dR_apply to take the per-node launch cost

@@ -698,3 +698,13 @@ def test_fc_sweep(lib, dev, oracle, C, H, W, N):
     got = dev.get(y, (N,))
     assert_close(got, want, terms=K)
     assert_close(got, oracle.fc_f64(x, Wt, b).reshape(-1), terms=K)
+
+
+def test_mfma_clock_probe(lib, gpu):
+    """The measurement aid of bench.py: shader clock under a stream of fp32 MFMAs, from the two clock counters a wave
+    can read.  Somewhere between idle clocks and the 2.4 GHz of the data sheet."""
+    mhz, us = ctypes.c_float(0), ctypes.c_float(0)
+    lib.drhip_mfma_clock_probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
+    ok(lib, lib.drhip_mfma_clock_probe(100, 3, ctypes.byref(mhz), ctypes.byref(us), None))
+    assert 500.0 < mhz.value < 2600.0 and us.value > 5.0, (mhz.value, us.value)
+    assert lib.drhip_mfma_clock_probe(0, 1, ctypes.byref(mhz), None, None) == -1
