@@ -240,10 +240,11 @@ def test_caller_stream_through_set_cl_environment(lib, dev, oracle):
 
 
 def test_debug_layer_download_and_profiling_switches(lib, dev, oracle, capfd):
-    """debugLayer + hostDebugBuffer: dR_apply copies the first channel plane (width x height floats, as the
-    reference does, src/deepRACIN.c:235-238) of the chosen layer into the caller's host array.  Set before
-    dR_prepare, the layer keeps a tensor of its own although a fusion would do away with it (the convolution in
-    front of a 2x2/2 max pool); set afterwards on such a layer, the pass says so and leaves the array alone.
+    """debugLayer: dR_apply copies the first channel plane (width x height floats, as the reference does,
+    src/deepRACIN.c:235-238) of the chosen layer into hostDebugBuffer, the host array the graph allocates for this at
+    dR_prepare and frees at dR_cleanup (src/dR_core.c:322,493).  Set before dR_prepare, the layer keeps a tensor of
+    its own although a fusion would do away with it (the convolution in front of a 2x2/2 max pool); set afterwards on
+    such a layer, the pass says so and leaves the array alone.
     profilingCPU: the pass is timed on the host and waited for; profilingGPU: per-node kernel times."""
     spec, feeds = small_spec(seed=6)
     want = oracle.run_spec(spec, feeds)
@@ -252,24 +253,25 @@ def test_debug_layer_download_and_profiling_switches(lib, dev, oracle, capfd):
             g, nodes = _graph(env, spec, [4])
             gs = dr.graph_struct(g)
             conv = dr.node_struct(nodes[1])
-            plane = np.full(spec[0]["shape"][0] * spec[0]["shape"][1], -1.0, np.float32)
             if early:
                 gs.debugLayer = conv.layerID
             dr.prepare(g)
+            assert gs.hostDebugBuffer                       # the graph's own array, large enough for its largest tensor
+            n = conv.oshape.s0 * conv.oshape.s1
+            plane = np.ctypeslib.as_array(ctypes.cast(gs.hostDebugBuffer, POINTER(c_float)), shape=(n,))
+            plane[:] = -1.0
             configs.feed_chw(nodes[0], feeds[0])
-            gs.hostDebugBuffer = plane.ctypes.data_as(c_void_p).value
             gs.debugLayer = conv.layerID
             capfd.readouterr()
             assert lib.dR_apply(g.ptr)
             (soft,) = configs.fetch_chw(g)
             assert_close(soft.reshape(-1), want[4].reshape(-1), "softmax of a pass with a debug download")
             if early:
-                assert_close(plane.reshape(conv.oshape.s1, conv.oshape.s0), want[1][0], "debug download of the convolution's first plane")
+                assert_close(plane.reshape(conv.oshape.s1, conv.oshape.s0).copy(), want[1][0], "debug download of the convolution's first plane")
                 continue
             assert np.all(plane == -1.0)
             assert "its tensor is never stored" in capfd.readouterr().out
             gs.debugLayer = -1
-            gs.hostDebugBuffer = None
             cfg = dr.graph_config(g)
             cfg.profilingCPU = 1
             capfd.readouterr()
@@ -285,6 +287,7 @@ def test_debug_layer_download_and_profiling_switches(lib, dev, oracle, capfd):
             assert lib.dR_apply(g.ptr)
             (soft,) = configs.fetch_chw(g)
             assert_close(soft.reshape(-1), want[4].reshape(-1), "softmax after the switches were turned off again")
+            del plane
 
 
 def test_compiled_c_host_program_classifies_the_reference_images(gpu, tmp_path):
