@@ -367,7 +367,9 @@ def _short(name):
 
 def _last_pass(rows, last=0):
     """Dispatches of the last complete forward pass: those after the second-to-last softmax launch up to the last
-    one; for workloads without a softmax the trailing `last` dispatches (all of them when `last` is 0)."""
+    one; for workloads without a softmax the trailing `last` dispatches (all of them when `last` is 0), the
+    runtime's own copy kernels (a synchronous read-back at the end of the run) not counted."""
+    rows = [r for r in rows if not r["kernel"].startswith("__amd_rocclr")]
     ends = [i for i, r in enumerate(rows) if "softmax" in r["kernel"]]
     if len(ends) >= 2 and not last:
         return rows[ends[-2] + 1: ends[-1] + 1]
@@ -503,6 +505,7 @@ def main():
     ap.add_argument("--no-secondary", action="store_true", help="skip the second network of the headline metric")
     ap.add_argument("--no-configs", action="store_true", help="skip the three small configurations")
     ap.add_argument("--layers", action="store_true", help="also print a per-layer table to stderr")
+    ap.add_argument("--no-clock-probe", action="store_true", help="skip the measurement of the shader clock under a stream of MFMAs (profile runs)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the workload, run 4 plain copies of 256 MiB (copy3d_kernel): under rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE their known traffic gives the scale of the counters")
@@ -540,7 +543,7 @@ def main():
     # clock of such a stream, measured now on this GPU, caps every utilisation figure against the data-sheet peak.
     mhz, probe_us = ctypes.c_float(0.0), ctypes.c_float(0.0)
     lib.drhip_mfma_clock_probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float), ctypes.c_void_p]
-    if lib.drhip_mfma_clock_probe(200, 500, ctypes.byref(mhz), ctypes.byref(probe_us), None) == 0 and mhz.value > 0 and roofline and "mfma_busy_frac" in roofline:
+    if not args.no_clock_probe and lib.drhip_mfma_clock_probe(200, 500, ctypes.byref(mhz), ctypes.byref(probe_us), None) == 0 and mhz.value > 0 and roofline and "mfma_busy_frac" in roofline:
         roofline["mfma_stream_clock_mhz"] = round(mhz.value, 1)
         roofline["mfma_stream_probe_us"] = round(probe_us.value, 1)
         roofline["mfma_busy_frac_at_stream_clock"] = round(roofline["mfma_busy_frac"] * PEAK_CLOCK_GHZ * 1e3 / mhz.value, 4)

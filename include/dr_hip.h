@@ -190,7 +190,7 @@ int drhip_conv3x3_winograd_f32(const float* in, const float* U, const float* bia
  * work-group search in dR_conv2d_winograd_schedule (src/dR_nodes_conv2d.c:809-1006). */
 int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O);
 size_t drhip_conv3x3_winograd_workspace_floats(int W, int H, int I, int O, int variant);
-/* Variants with bit 0x800 ("joined splits": 32-tile blocks, 2, 4 or 8 equal input-channel splits, all workgroups
+/* Variants with bit 0x800 ("joined splits": 32-tile blocks, 2, 4, 8 or 16 equal input-channel splits, all workgroups
  * of the launch resident at once) add the splits' partial tiles up inside the one launch instead of in a second
  * kernel: every split finishes a slice of its panel and recognises a partial tile that has not arrived yet by the
  * marker value its workspace slot still holds.  The workspace of such a variant has to go through
@@ -200,6 +200,11 @@ size_t drhip_conv3x3_winograd_workspace_floats(int W, int H, int I, int O, int v
  * not deliver within the kernel's bounded wait (about 0.2 s: the device was shared so that the launch was not
  * resident as a whole) turns the affected outputs into NaN and is counted; drhip_conv3x3_winograd_join_timeouts
  * reads that count (a synchronous copy).  Environment DR_WINO_JOIN=0 keeps pick_variant from returning such variants.
+ * Bit 0x1000 on top of 0x800 ("tiered", four waves, 32 or 64 channels per workgroup, split bits zero) lets the
+ * launcher cut a layer whose blocks do not divide by the compute units into tiers: as many whole blocks per unit as fit,
+ * then the rest halved, quartered ... over the input channels (joined as above) so that every unit gets the same
+ * number of channel stages; the number of splits then differs per block and is not the caller's to choose.
+ * Environment DR_WINO_TIERS=0 keeps pick_variant from returning it.
  * No counterpart in the reference: its kernel never splits the channel sum (Kernels/dR_winograd2.cl:176-189). */
 int drhip_conv3x3_winograd_workspace_prepare_f32(float* workspace, size_t floats, void* stream);
 int drhip_conv3x3_winograd_join_timeouts(unsigned* count);
