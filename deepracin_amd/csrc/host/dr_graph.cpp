@@ -247,10 +247,13 @@ void dR_feedData(dR_Graph* net, dR_Node* feednode, gfloat* data, gint offset, gi
 }
 
 // One forward pass: walks the schedule and lets every node enqueue its kernels.  Asynchronous
-// unless profiling is enabled (reference src/deepRACIN.c:204-270: clFlush only).  The first plain
-// pass records the node walk into a hipGraph; later passes replay it with a single launch.
-// DR_HIPGRAPH=0 in the environment, profilingGPU, a debug layer, or a node whose compute() cannot
-// be captured (it blocks or allocates) keep the node-by-node path.
+// unless profiling is enabled (reference src/deepRACIN.c:204-270: clFlush only).  With DR_HIPGRAPH=1
+// in the environment the first plain pass records the node walk into a hipGraph and later passes
+// replay it with a single launch (not with profilingGPU, a debug layer, or a node whose compute()
+// cannot be captured because it blocks or allocates).  Off by default: enqueueing a node costs the
+// host 2.5-3 us, less than the shortest kernels take, and kernels enqueued one by one follow each
+// other more closely on the device than the kernel nodes of a replayed graph (SqueezeNet 81.8 against
+// 87.5 us per pass, VGG16 287.2 against 291.4 us, first result of a single pass 8 us sooner).
 //
 // profilingGPU: the reference waits for every kernel and reads its cl_event (src/dR_clwrap.c:970-1049).
 // Here every kernel launch of the pass carries its own start/stop events while the pass is enqueued
@@ -280,12 +283,12 @@ gboolean dR_apply(dR_Graph* net) {
     std::chrono::steady_clock::time_point t0;
     if (profCPU) { t0 = std::chrono::steady_clock::now(); net->config->totalNodeCPUTime = 0.0; }
 
-    // Plain passes are replayed from a hipGraph captured on the first one: at batch 1 the nodes are
-    // so short that enqueueing them one by one costs more host time than they take to run.
+    // On request plain passes are replayed from a hipGraph captured on the first one (for hosts too slow or
+    // too busy to enqueue a node in the time the device takes to run it).
     if (!profGPU && net->debugLayer < 0 && !net->drGraphOff) {
         if (!net->drGraphExec) {
             const char* env = getenv("DR_HIPGRAPH");
-            if ((env && strcmp(env, "0") == 0) || drhip_graph_capture_begin(cc->hipStream) != DRHIP_OK) {
+            if (!env || strcmp(env, "1") != 0 || drhip_graph_capture_begin(cc->hipStream) != DRHIP_OK) {
                 net->drGraphOff = TRUE;
             } else {
                 const bool recorded = record_forward_pass(net);

@@ -180,7 +180,7 @@ struct dR_Graph {
     dR_List*        drViewHandlers;         /* handlers that alias a slice of a stream buffer */
     gdouble         drLastApplyMs;          /* wall ms of the last dR_apply when profilingCPU */
     void*           drGraphExec;            /* hipGraphExec_t of the captured forward pass, NULL until captured */
-    gboolean        drGraphOff;             /* TRUE: always enqueue node by node (capture failed or DR_HIPGRAPH=0) */
+    gboolean        drGraphOff;             /* TRUE: always enqueue node by node (DR_HIPGRAPH=1 not set, or capture failed) */
     void*           drSideStreams[3];       /* streams that carry independent sibling nodes inside the captured graph */
     void*           drBranchEvents[4];      /* fork event [0] and join events [1..3] of a sibling group */
     gint            drBranchGroups;         /* number of sibling groups the captured graph runs concurrently */

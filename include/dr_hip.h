@@ -77,8 +77,8 @@ int drhip_stream_wait_event(void* stream, void* ev);      /* later work on `stre
 int drhip_mfma_clock_probe(int iters, int launches, float* mhz_median, float* microseconds, void* stream);
 
 /* ---- launch graphs: record everything enqueued on `stream` between begin and end into an executable
- *      hipGraph and replay it with one call.  Used by dR_apply to take the per-node launch cost
- *      (dozens of small kernels at batch 1) off the host.  capture_end returns DRHIP_EDEVICE and a NULL
+ *      hipGraph and replay it with one call.  dR_apply uses it on request (DR_HIPGRAPH=1) to take the
+ *      per-node launch cost (dozens of small kernels at batch 1) off the host.  capture_end returns DRHIP_EDEVICE and a NULL
  *      graph if something that cannot be captured (a blocking call, an allocation) happened in
  *      between; the stream is usable again afterwards. */
 int drhip_graph_capture_begin(void* stream);
