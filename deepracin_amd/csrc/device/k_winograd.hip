@@ -971,7 +971,9 @@ extern "C" int drhip_conv3x3_winograd_pick_variant(int W, int H, int I, int O) {
     if (ceil_div(T, 32) * ceil_div(O, 32) < cus / 2 && ceil_div(I, kWinoKC) <= 16)
         // 6+ stages and at most one workgroup per CU (14x14 maps; 56x56 64->64: 5.3 vs 5.5 us): two wave sets
         return (ceil_div(I, kWinoKC) >= 6 && ceil_div(T, 16) * ceil_div(O, 16) <= cus) ? 0x501 : 0x101;
-    const int code = (O > 32 && T >= 8192) ? 2 : 1;
+    // (an image layer has next to no transform work to share, and twice the workgroups of half the size spread its
+    // stores better: 224x224 3->64 6.1 vs 6.7 us)
+    const int code = (O > 32 && T >= 8192 && I > 4) ? 2 : 1;
     const int panels = ceil_div(T, 32) * ceil_div(O, code == 2 ? 64 : 32);
     const int nChunks = ceil_div(I, kWinoKC);
     int lg = 0;

@@ -312,7 +312,9 @@ def test_winograd_tiered_refused_combinations(lib, dev):
 def test_winograd_auto_variant_vgg_shapes(lib, dev, oracle):
     assert lib.drhip_conv3x3_winograd_pick_variant(112, 112, 128, 128) == 0x1801      # (MI355X: 32 CUs per XCD)
     assert lib.drhip_conv3x3_winograd_pick_variant(14, 14, 512, 512) == 0x831
-    for (W, I, O) in [(224, 64, 64), (112, 128, 128), (56, 128, 256), (28, 256, 512), (14, 512, 512)]:
+    assert lib.drhip_conv3x3_winograd_pick_variant(224, 224, 3, 64) == 1           # an image layer: 32-channel blocks
+    assert lib.drhip_conv3x3_winograd_pick_variant(224, 224, 64, 64) == 2
+    for (W, I, O) in [(224, 3, 64), (224, 64, 64), (112, 128, 128), (56, 128, 256), (28, 256, 512), (14, 512, 512)]:
         x, w, b = np.abs(rnd(I, W, W)), rnd(I, O, 3, 3, scale=np.sqrt(2.0 / (9 * I))), rnd(O, scale=0.01)
         U, _ = wino_filters(lib, dev, w)
         variant = lib.drhip_conv3x3_winograd_pick_variant(W, W, I, O)
