@@ -92,7 +92,7 @@ __device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {
     const float* pp = d.partials + row;
     float s = 0.0f;
     int sl = 0;
-    // 32, then 8 independent loads in flight, always summed in slice order: the partial sums come
+    // 32, 16, then 8 independent loads in flight, always summed in slice order: the partial sums come
     // from other XCDs' workgroups, so every round of loads costs a trip to memory
     for (; sl + 32 <= d.slices; sl += 32) {
         float v[32];
@@ -100,6 +100,13 @@ __device__ inline float deferred_element(const drhip_deferred_vec& d, int row) {
         for (int u = 0; u < 32; ++u) v[u] = pp[(size_t)(sl + u) * d.n];
 #pragma unroll
         for (int u = 0; u < 32; ++u) s += v[u];
+    }
+    for (; sl + 16 <= d.slices; sl += 16) {         // (a GEMV that fills the chip leaves 16 slices: one round, not two)
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = pp[(size_t)(sl + u) * d.n];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) s += v[u];
     }
     for (; sl < d.slices; sl += 8) {                // the ragged end too: clamped loads, zeros by select
         float v[8];
