@@ -160,15 +160,27 @@ def measure(workload, seed, steps, warmup, blocks=BLOCKS, instrument=True, env_v
                "launch_graph": bool(dr.graph_struct(g).drGraphExec)}
 
         # wall-clock rate of the loop the reference's users run: feed (H2D over PCIe), pass, download of the output
+        # (the three C calls with buffers set up once, as a C caller has them: no array is created inside the loop)
         feed_idx, feed_arr = next(iter(feeds.items()))
+        feed_arr = np.ascontiguousarray(feed_arr, np.float32)
+        feed_ptr, feed_node = feed_arr.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), nodes[feed_idx].ptr
+        mem = (dr.c_void_p * max(g.num_outputs, 1))()
+        n_out = lib.dR_getOutputBuffers(g.ptr, mem)
+        host = [np.empty(int(np.prod(g.outnodes[i].out_shape)), np.float32) for i in range(n_out)]
+        host_ptr = [h.ctypes.data_as(dr.c_void_p) for h in host]
+
+        def one_round():
+            lib.dR_feedData(g.ptr, feed_node, feed_ptr, 0, feed_arr.size)
+            lib.dR_apply(g.ptr)
+            for i in range(n_out):
+                lib.dR_downloadArray(g.ptr, b"output", mem[i], 0, host[i].nbytes, host_ptr[i])
+
         n_e2e = max(steps, 100)
         for _ in range(3):
-            configs.feed_chw(nodes[feed_idx], feed_arr); lib.dR_apply(g.ptr); configs.fetch_chw(g)
+            one_round()
         t0 = time.perf_counter()
         for _ in range(n_e2e):
-            configs.feed_chw(nodes[feed_idx], feed_arr)
-            lib.dR_apply(g.ptr)
-            configs.fetch_chw(g)
+            one_round()
         res["e2e_ms"] = (time.perf_counter() - t0) * 1e3 / n_e2e
 
         if instrument:
