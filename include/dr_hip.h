@@ -95,12 +95,15 @@ int drhip_download(void* dst_host, const void* src_dev, size_t src_byte_offset, 
 int drhip_fill_f32(float* dst, float value, size_t n, void* stream);
 /* Staged transfers for the per-image copies of a serving loop (the feed of dR_feedData, the logits of
  * dR_downloadArray).  A staging object owns pinned host memory (hipHostMalloc): an upload area of
- * `upload_bytes` and a 64 KiB download area.  drhip_upload_staged copies the caller's (pageable) array
- * into the upload area and starts one transfer from there (up to 4 MiB: a kernel that reads the pinned
+ * `upload_bytes` (two of them, used in turn) and a 64 KiB download area.  drhip_upload_staged copies the caller's (pageable) array
+ * into an upload area and starts one transfer from there (up to 4 MiB: a kernel that reads the pinned
  * area, which starts sooner than the DMA engine; DR_UPLOAD_KERNEL=0 in the environment or larger arrays:
  * hipMemcpyAsync); it returns when the caller's array has been
  * read (the array may be reused), NOT when the data is on the device: the transfer is ordered on
- * `stream` before whatever is enqueued next, and a following staged upload waits for it.
+ * `stream` before whatever is enqueued next.  An area is written again two uploads later; that the upload which
+ * read it has finished follows from any staged download that completed on the same stream in between (the usual
+ * feed / pass / download loop: nothing is recorded, nothing waited for); a caller that uploads again before any
+ * download has completed gets an event recorded behind its upload, which the upload after the next waits for.
  * drhip_download_staged blocks like drhip_download; the data comes through the download area, stored
  * there by a small copy kernel (the area is mapped into the device's address space) that raises a flag
  * behind the data; the host watches the flag for up to DR_SPIN_US microseconds (default 1000; 0 = never)

@@ -560,6 +560,20 @@ def test_staged_transfers_carry_every_byte(lib, dev, env):
             back = np.full(n, -1.0, np.float32)
             ok(lib, lib.drhip_download_staged(h, back.ctypes.data_as(vp), buf, 4 * off, back.nbytes, None))
             assert np.array_equal(back, a_copy), (it, n, off)
+        # many uploads in a row with no download in between (the two pinned areas are reused while earlier uploads
+        # may still be in flight), the caller's array overwritten after every call
+        n, rows = 4096, 24
+        src = np.empty(n, np.float32)
+        want = np.empty((rows, n), np.float32)
+        for k in range(rows):
+            src[...] = rng.standard_normal(n).astype(np.float32) + 100 * k
+            want[k] = src
+            ok(lib, lib.drhip_upload_staged(h, buf, 4 * k * n, src.ctypes.data_as(vp), src.nbytes, None))
+            src[...] = np.nan
+        for k in range(rows):
+            back = np.full(n, -1.0, np.float32)
+            ok(lib, lib.drhip_download_staged(h, back.ctypes.data_as(vp), buf, 4 * k * n, back.nbytes, None))
+            assert np.array_equal(back, want[k]), k
         # bytes that are not whole floats go through the DMA engine both ways
         raw = rng.integers(0, 256, 1001, dtype=np.uint8)
         ok(lib, lib.drhip_upload_staged(h, buf, 3, raw.ctypes.data_as(vp), raw.nbytes, None))
