@@ -361,18 +361,25 @@ int drhip_upload_staged(void* handle, void* dst, size_t off, const void* src, si
         } else if (int rc = check(hipStreamSynchronize(area.stream), "hipStreamSynchronize(staging)")) return rc;
         area.pending = area.recorded = false;
     }
-    // One piece: splitting the array so that the host copy of one piece overlaps the transfer of the one before
-    // was measured slower (0.414 vs 0.386 ms per VGG16 image with 128 KiB pieces: every transfer call costs the
-    // host more than the overlap returns).
-    memcpy(area.mem, src, bytes);
     // A few hundred KiB: a kernel that reads the pinned area over the bus starts sooner than the DMA engine
-    // (602 KB image: 4 us less per pass).
+    // (602 KB image: 4 us less per pass).  From 256 KiB on in two pieces: the kernel of the first half runs while
+    // the host copies the second (2 us less per 602 KB image; with five pieces moved by the DMA engine the calls cost
+    // the host more than the overlap returned, 0.414 vs 0.386 ms per VGG16 image).
     if (s->uploadByKernel && bytes <= kStagingKernelUpload && ((size_t)((char*)dst + off) % 16 == 0) && bytes % 4 == 0) {
-        const size_t n = bytes / 4, n4 = n / 4;
-        launch(copy_from_host_kernel, dim3((unsigned)std::max<size_t>(1, std::min<size_t>((n4 + 255) / 256, 512))), dim3(256), 0, as_stream(stream),
-               (float*)((char*)dst + off), (const float*)area.mem, n4, n);
-        if (int rc = launched("copy_from_host_kernel")) return rc;
-    } else if (int rc = check(hipMemcpyAsync((char*)dst + off, area.mem, bytes, hipMemcpyHostToDevice, as_stream(stream)), "hipMemcpyAsync(H2D, staged)")) return rc;
+        const size_t first = bytes >= (256u << 10) ? (bytes / 2) & ~(size_t)15 : bytes;
+        const size_t begins[2] = {0, first}, lens[2] = {first, bytes - first};
+        for (int piece = 0; piece < 2 && lens[piece] > 0; ++piece) {
+            const size_t begin = begins[piece], len = lens[piece];
+            memcpy(area.mem + begin, (const char*)src + begin, len);
+            const size_t n = len / 4, n4 = n / 4;
+            launch(copy_from_host_kernel, dim3((unsigned)std::max<size_t>(1, std::min<size_t>((n4 + 255) / 256, 512))), dim3(256), 0, as_stream(stream),
+                   (float*)((char*)dst + off + begin), (const float*)(area.mem + begin), n4, n);
+            if (int rc = launched("copy_from_host_kernel")) return rc;
+        }
+    } else {
+        memcpy(area.mem, src, bytes);
+        if (int rc = check(hipMemcpyAsync((char*)dst + off, area.mem, bytes, hipMemcpyHostToDevice, as_stream(stream)), "hipMemcpyAsync(H2D, staged)")) return rc;
+    }
     area.pending = true;
     area.recorded = false;
     area.stream = as_stream(stream);
